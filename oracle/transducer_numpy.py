@@ -1,0 +1,420 @@
+"""CPU oracle for the RNNT / TDT transducer loss -- TEST INFRASTRUCTURE ONLY.
+
+Nothing in the shipped package may import this module.  It is a plain
+numpy restatement (per-cell Python loops, float64 by default) of what the
+reference computes on its GPU path, written from the recursions and not from
+the reference source.  Each function names the reference lines it restates
+(paths relative to nemo/collections/asr/parts/numba/rnnt_loss/).
+
+How each function is pinned (tests/test_oracle_*.py):
+  denominator       closed form -logsumexp (scipy) .................. pinned
+  lse2              reference KAT log_sum_exp(0,1)*8=10.5060935 ...... pinned
+  rnnt_*            reference golden vectors small / small_blank_last /
+                    medium (cost + full gradient), clamp vector,
+                    FastEmit cost scaling, brute-force path enumeration,
+                    torch autograd of an alpha-only recursion ........ pinned
+  tdt_*             reference fixed vector (cost 4.155739 + 42 grads),
+                    brute-force (token,duration) path enumeration,
+                    torch autograd, T=1 and U=1 closed forms ......... pinned
+  tdt_* FastEmit    no reference vector exists; checked only against the
+                    sparse-posterior + softmax-Jacobian identity ..... derived
+
+The loops are slow on purpose (clarity first): use them at lattice sizes up to
+a few thousand cells; oracle/transducer_cpu.c is the fast restatement.
+"""
+
+import numpy as np
+
+NEG_INF = -np.inf
+# utils/cuda_utils/gpu_rnnt_kernel.py:38 -- the TDT kernels seed their
+# accumulators with a finite sentinel, not with -inf.
+TDT_NEG = -10000.0
+
+
+def lse2(a, b):
+    """log(exp(a)+exp(b)); utils/rnnt_helper.py:42-53.
+
+    Returns the other operand untouched when one of them is exactly -inf.
+    """
+    if a == NEG_INF:
+        return b
+    if b == NEG_INF:
+        return a
+    if a > b:
+        return np.log1p(np.exp(b - a)) + a
+    return np.log1p(np.exp(a - b)) + b
+
+
+def denominator(acts):
+    """denom[...] = -max_v x - log sum_v exp(x - max).
+
+    utils/cuda_utils/reduce.py:121-248 driven by
+    utils/cuda_utils/gpu_rnnt.py:93-123 (max pass, then sum-exp pass with
+    the sign flipped).
+    """
+    m = acts.max(axis=-1)
+    s = np.exp(acts - m[..., None]).sum(axis=-1)
+    return -m - np.log(s)
+
+
+# ----------------------------------------------------------------------------
+# RNNT (utils/cuda_utils/gpu_rnnt_kernel.py:73-407)
+# ----------------------------------------------------------------------------
+
+
+def rnnt_alphas(lp, labels, T, U, blank):
+    """Forward variables; gpu_rnnt_kernel.py:73-172.
+
+    lp: [>=T, >=U, V] log-probabilities (logits + denominator).
+    labels: at least U-1 label ids.  Returns (alphas[T,U], ll_forward).
+    """
+    dt = lp.dtype.type
+    a = np.full((T, U), NEG_INF, dtype=lp.dtype)
+    a[0, 0] = dt(0)
+    for t in range(T):
+        for u in range(U):
+            if t == 0 and u == 0:
+                continue
+            if u == 0:
+                a[t, 0] = a[t - 1, 0] + lp[t - 1, 0, blank]
+            elif t == 0:
+                a[0, u] = a[0, u - 1] + lp[0, u - 1, labels[u - 1]]
+            else:
+                no_emit = a[t - 1, u] + lp[t - 1, u, blank]
+                emit = a[t, u - 1] + lp[t, u - 1, labels[u - 1]]
+                a[t, u] = lse2(emit, no_emit)
+    ll = a[T - 1, U - 1] + lp[T - 1, U - 1, blank]
+    return a, ll
+
+
+def rnnt_betas(lp, labels, T, U, blank):
+    """Backward variables; gpu_rnnt_kernel.py:175-269.  Returns (betas, betas[0,0])."""
+    b = np.full((T, U), NEG_INF, dtype=lp.dtype)
+    b[T - 1, U - 1] = lp[T - 1, U - 1, blank]
+    for t in range(T - 1, -1, -1):
+        for u in range(U - 1, -1, -1):
+            if t == T - 1 and u == U - 1:
+                continue
+            if u == U - 1:
+                b[t, u] = b[t + 1, u] + lp[t, u, blank]
+            elif t == T - 1:
+                b[t, u] = b[t, u + 1] + lp[t, u, labels[u]]
+            else:
+                no_emit = b[t + 1, u] + lp[t, u, blank]
+                emit = b[t, u + 1] + lp[t, u, labels[u]]
+                b[t, u] = lse2(emit, no_emit)
+    return b, b[0, 0]
+
+
+def rnnt_grads(lp, alphas, betas, ll, labels, T, U, blank, fastemit_lambda, clamp):
+    """Gradient of the cost w.r.t. the logits; gpu_rnnt_kernel.py:272-407.
+
+    Same term order as the kernel: the dense exp(alpha+beta+lp-ll) term, the
+    FastEmit addition, the three sparse subtractions, then the clamp.
+    """
+    dt = lp.dtype.type
+    V = lp.shape[-1]
+    g = np.zeros((T, U, V), dtype=lp.dtype)
+    lam = dt(fastemit_lambda)
+    for t in range(T):
+        for u in range(U):
+            row = np.exp(alphas[t, u] + betas[t, u] + lp[t, u, :] - ll)
+            if fastemit_lambda > 0.0 and u < U - 1:
+                row = row + lam * np.exp(
+                    alphas[t, u] + lp[t, u, labels[u]] + betas[t, u + 1] + lp[t, u, :] - ll
+                )
+            if t == T - 1 and u == U - 1:
+                row[blank] -= np.exp(alphas[t, u] + lp[t, u, blank] - ll)
+            if t < T - 1:
+                row[blank] -= np.exp(alphas[t, u] + lp[t, u, blank] - ll + betas[t + 1, u])
+            if u < U - 1:
+                v = labels[u]
+                row[v] -= np.exp(np.log1p(lam) + alphas[t, u] + lp[t, u, v] - ll + betas[t, u + 1])
+            if clamp > 0.0:
+                row = np.minimum(np.maximum(row, dt(-clamp)), dt(clamp))
+            g[t, u, :] = row
+    return g
+
+
+def rnnt_loss(acts, labels, act_lens, label_lens, blank, fastemit_lambda=0.0, clamp=0.0, dtype=np.float64):
+    """Per-utterance costs and logits-gradient for a padded batch.
+
+    Restates GPURNNT.compute_cost_and_score (utils/cuda_utils/gpu_rnnt.py:125-231)
+    plus compute_costs_data (utils/rnnt_helper.py:106-116): cost = -ll*(1+lambda),
+    padded cells get a zero gradient.  `acts` are raw logits [B,T,U,V].
+    Returns (costs[B], grads[B,T,U,V], extras) with extras holding denom,
+    alphas, betas (padded with -inf outside the valid lattice), ll_forward, ll_backward.
+    """
+    acts = np.asarray(acts, dtype=dtype)
+    B, Tm, Um, V = acts.shape
+    denom = denominator(acts)
+    costs = np.zeros(B, dtype=dtype)
+    grads = np.zeros_like(acts)
+    alphas = np.full((B, Tm, Um), NEG_INF, dtype=dtype)
+    betas = np.full((B, Tm, Um), NEG_INF, dtype=dtype)
+    llf = np.zeros(B, dtype=dtype)
+    llb = np.zeros(B, dtype=dtype)
+    for b in range(B):
+        T = int(act_lens[b])
+        U = int(label_lens[b]) + 1
+        lp = acts[b] + denom[b][..., None]
+        lab = [int(x) for x in labels[b][: U - 1]]
+        a, ll = rnnt_alphas(lp, lab, T, U, blank)
+        bt, ll_b = rnnt_betas(lp, lab, T, U, blank)
+        grads[b, :T, :U, :] = rnnt_grads(lp, a, bt, ll, lab, T, U, blank, fastemit_lambda, clamp)
+        alphas[b, :T, :U] = a
+        betas[b, :T, :U] = bt
+        llf[b], llb[b] = ll, ll_b
+        costs[b] = -ll * dtype(1.0 + fastemit_lambda)
+    return costs, grads, dict(denom=denom, alphas=alphas, betas=betas, ll_forward=llf, ll_backward=llb)
+
+
+# ----------------------------------------------------------------------------
+# TDT (utils/cuda_utils/gpu_rnnt_kernel.py:888-1439)
+# ----------------------------------------------------------------------------
+
+
+def tdt_alphas(lp, dlp, labels, T, U, blank, durations, sigma):
+    """TDT forward variables; gpu_rnnt_kernel.py:888-1073.
+
+    lp: token log-probs [.,.,V]; dlp: duration log-probs [.,.,D]; durations ascending.
+    """
+    dt = lp.dtype.type
+    sig = dt(sigma)
+    NEG = dt(TDT_NEG)
+    D = len(durations)
+    a = np.full((T, U), NEG_INF, dtype=lp.dtype)
+    a[0, 0] = dt(0)
+    for t in range(T):
+        for u in range(U):
+            if t == 0 and u == 0:
+                continue
+            if u == 0:
+                acc = NEG
+                for i in range(D):
+                    d = durations[i]
+                    if d == 0:
+                        continue
+                    if t >= d:
+                        acc = lse2(acc, a[t - d, 0] + lp[t - d, 0, blank] - sig + dlp[t - d, 0, i])
+                    else:
+                        break
+                a[t, 0] = acc
+            elif t == 0:
+                if durations[0] == 0:
+                    a[0, u] = a[0, u - 1] + lp[0, u - 1, labels[u - 1]] - sig + dlp[0, u - 1, 0]
+                else:
+                    a[0, u] = NEG
+            else:
+                no_emit = NEG
+                for i in range(D):
+                    d = durations[i]
+                    if d == 0:
+                        continue
+                    if t >= d:
+                        no_emit = lse2(no_emit, a[t - d, u] + lp[t - d, u, blank] - sig + dlp[t - d, u, i])
+                    else:
+                        break
+                emit = NEG
+                for i in range(D):
+                    d = durations[i]
+                    if t >= d:
+                        emit = lse2(emit, a[t - d, u - 1] + lp[t - d, u - 1, labels[u - 1]] - sig + dlp[t - d, u - 1, i])
+                    else:
+                        break
+                a[t, u] = lse2(emit, no_emit)
+    ll = NEG
+    for i in range(D):
+        d = durations[i]
+        if d == 0:
+            continue
+        if d == 1:
+            # assigned, not accumulated (gpu_rnnt_kernel.py:1054-1061)
+            ll = a[T - 1, U - 1] + lp[T - 1, U - 1, blank] - sig + dlp[T - 1, U - 1, i]
+            continue
+        if T >= d:
+            ll = lse2(ll, a[T - d, U - 1] + lp[T - d, U - 1, blank] - sig + dlp[T - d, U - 1, i])
+        else:
+            break
+    return a, ll
+
+
+def tdt_betas(lp, dlp, labels, T, U, blank, durations, sigma):
+    """TDT backward variables; gpu_rnnt_kernel.py:1076-1241."""
+    dt = lp.dtype.type
+    sig = dt(sigma)
+    NEG = dt(TDT_NEG)
+    D = len(durations)
+    b = np.full((T, U), NEG_INF, dtype=lp.dtype)
+    # the duration-1 index is looked for at positions 0 and 1 only (:1137-1148)
+    if durations[0] == 1:
+        b[T - 1, U - 1] = lp[T - 1, U - 1, blank] - sig + dlp[T - 1, U - 1, 0]
+    elif D > 1 and durations[1] == 1:
+        b[T - 1, U - 1] = lp[T - 1, U - 1, blank] - sig + dlp[T - 1, U - 1, 1]
+    else:
+        raise ValueError("TDT durations must hold 1 at position 0 or 1")
+    for t in range(T - 1, -1, -1):
+        for u in range(U - 1, -1, -1):
+            if t == T - 1 and u == U - 1:
+                continue
+            if u == U - 1:
+                acc = NEG
+                for i in range(D):
+                    d = durations[i]
+                    if d == 0:
+                        continue
+                    if t + d < T:
+                        acc = lse2(acc, b[t + d, u] + lp[t, u, blank] + dlp[t, u, i] - sig)
+                    elif t + d == T:
+                        acc = lse2(acc, lp[t, u, blank] + dlp[t, u, i] - sig)
+                b[t, u] = acc
+            elif t == T - 1:
+                if durations[0] == 0:
+                    b[t, u] = b[t, u + 1] + lp[t, u, labels[u]] + dlp[t, u, 0] - sig
+                else:
+                    b[t, u] = NEG
+            else:
+                no_emit = NEG
+                for i in range(D):
+                    d = durations[i]
+                    if d == 0:
+                        continue
+                    if t + d < T:
+                        no_emit = lse2(no_emit, b[t + d, u] + lp[t, u, blank] + dlp[t, u, i] - sig)
+                emit = NEG
+                for i in range(D):
+                    d = durations[i]
+                    if t + d < T:
+                        emit = lse2(emit, b[t + d, u + 1] + lp[t, u, labels[u]] + dlp[t, u, i] - sig)
+                b[t, u] = lse2(emit, no_emit)
+    return b, b[0, 0]
+
+
+def tdt_grads(lp, dlp, alphas, betas, ll, labels, T, U, blank, durations, sigma, fastemit_lambda, clamp):
+    """TDT gradients; gpu_rnnt_kernel.py:1244-1439.
+
+    Returns (label_grads[T,U,V] w.r.t. token logits, duration_grads[T,U,D]
+    w.r.t. duration LOG-PROBS -- the reference leaves the log-softmax Jacobian
+    of the duration branch to torch autograd, rnnt_pytorch.py:564-568).
+    """
+    dt = lp.dtype.type
+    sig = dt(sigma)
+    lam = dt(fastemit_lambda)
+    D = len(durations)
+    V = lp.shape[-1]
+    lg = np.zeros((T, U, V), dtype=lp.dtype)
+    dg = np.zeros((T, U, D), dtype=lp.dtype)
+    for t in range(T):
+        for u in range(U):
+            lpk_blank = lp[t, u, blank] - sig
+            for i in range(D):
+                d = durations[i]
+                g = dt(0)
+                if t + d < T and u < U - 1:
+                    lpk_label = lp[t, u, labels[u]] - sig
+                    g -= np.exp(alphas[t, u] + betas[t + d, u + 1] + lpk_label - ll)
+                if t + d < T and d > 0:
+                    g -= np.exp(alphas[t, u] + betas[t + d, u] + lpk_blank - ll)
+                if t + d == T and u == U - 1 and d > 0:
+                    g -= np.exp(alphas[t, u] + lpk_blank - ll)
+                dg[t, u, i] = g * np.exp(dlp[t, u, i])
+
+            row = np.exp(alphas[t, u] + betas[t, u] + lp[t, u, :] - ll)
+            if fastemit_lambda > 0.0 and u < U - 1:
+                fe = np.zeros(V, dtype=lp.dtype)
+                for i in range(D):
+                    d = durations[i]
+                    if t + d < T:
+                        fe = fe + lam * np.exp(
+                            alphas[t, u]
+                            + lp[t, u, labels[u]]
+                            + dlp[t, u, i]
+                            + betas[t + d, u + 1]
+                            + lp[t, u, :]
+                            - sig
+                            - ll
+                        )
+                row = row + fe
+            if u == U - 1:
+                for i in range(D):
+                    d = durations[i]
+                    if d == 0:
+                        continue
+                    if t == T - d:
+                        row[blank] -= np.exp(alphas[t, u] + lp[t, u, blank] - sig - ll + dlp[t, u, i])
+            for i in range(D):
+                d = durations[i]
+                if d == 0:
+                    continue
+                if t < T - d:
+                    row[blank] -= np.exp(alphas[t, u] + lp[t, u, blank] - sig - ll + betas[t + d, u] + dlp[t, u, i])
+            if u < U - 1:
+                v = labels[u]
+                for i in range(D):
+                    d = durations[i]
+                    if t + d < T:
+                        row[v] -= np.exp(
+                            np.log1p(lam) + alphas[t, u] + lp[t, u, v] - sig - ll + betas[t + d, u + 1] + dlp[t, u, i]
+                        )
+            if clamp > 0.0:
+                row = np.minimum(np.maximum(row, dt(-clamp)), dt(clamp))
+            lg[t, u, :] = row
+    return lg, dg
+
+
+def tdt_loss(
+    acts, labels, act_lens, label_lens, blank, durations, sigma=0.0, fastemit_lambda=0.0, clamp=0.0, dtype=np.float64
+):
+    """TDT costs and the gradient w.r.t. the COMBINED logits [B,T,U,V+D].
+
+    Restates TDTLossNumba.forward (rnnt_pytorch.py:554-583: split, token part
+    passed un-normalised, duration part log-softmaxed) + GPUTDT with omega = 0
+    (utils/cuda_utils/gpu_rnnt.py:563-743) + the autograd of that duration
+    log-softmax: dlogit_i = dg_i - softmax_i * sum_j dg_j.
+    Returns (costs[B], grads[B,T,U,V+D], extras).
+    """
+    acts = np.asarray(acts, dtype=dtype)
+    durations = [int(d) for d in durations]
+    D = len(durations)
+    B, Tm, Um, VD = acts.shape
+    V = VD - D
+    tok = acts[..., :V]
+    dur = acts[..., V:]
+    denom = denominator(tok)
+    dlp_all = dur + denominator(dur)[..., None]
+    costs = np.zeros(B, dtype=dtype)
+    grads = np.zeros_like(acts)
+    label_grads = np.zeros((B, Tm, Um, V), dtype=dtype)
+    duration_grads = np.zeros((B, Tm, Um, D), dtype=dtype)
+    alphas = np.full((B, Tm, Um), NEG_INF, dtype=dtype)
+    betas = np.full((B, Tm, Um), NEG_INF, dtype=dtype)
+    llf = np.zeros(B, dtype=dtype)
+    llb = np.zeros(B, dtype=dtype)
+    for b in range(B):
+        T = int(act_lens[b])
+        U = int(label_lens[b]) + 1
+        lp = tok[b] + denom[b][..., None]
+        dlp = dlp_all[b]
+        lab = [int(x) for x in labels[b][: U - 1]]
+        a, ll = tdt_alphas(lp, dlp, lab, T, U, blank, durations, sigma)
+        bt, ll_b = tdt_betas(lp, dlp, lab, T, U, blank, durations, sigma)
+        lg, dg = tdt_grads(lp, dlp, a, bt, ll, lab, T, U, blank, durations, sigma, fastemit_lambda, clamp)
+        label_grads[b, :T, :U] = lg
+        duration_grads[b, :T, :U] = dg
+        grads[b, :T, :U, :V] = lg
+        grads[b, :T, :U, V:] = dg - np.exp(dlp[:T, :U]) * dg.sum(axis=-1, keepdims=True)
+        alphas[b, :T, :U] = a
+        betas[b, :T, :U] = bt
+        llf[b], llb[b] = ll, ll_b
+        costs[b] = -ll * dtype(1.0 + fastemit_lambda)
+    extras = dict(
+        denom=denom,
+        dlp=dlp_all,
+        alphas=alphas,
+        betas=betas,
+        ll_forward=llf,
+        ll_backward=llb,
+        label_grads=label_grads,
+        duration_grads=duration_grads,
+    )
+    return costs, grads, extras
