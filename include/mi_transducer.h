@@ -1,0 +1,133 @@
+/* mi_transducer.h -- C ABI of the MI355X (gfx950) transducer-loss library.
+ *
+ * One shared library, libmi_transducer.so, replaces everything the reference
+ * runs below its function-level seam (nemo/collections/asr/parts/numba/rnnt_loss/):
+ *   rnnt.py:138-236  rnnt_loss_gpu      -> mi_rnnt_loss  (or mi_rnnt_forward + mi_rnnt_backward)
+ *   rnnt.py:239-363  tdt_loss_gpu       -> mi_tdt_loss   (or mi_tdt_forward  + mi_tdt_backward)
+ *   utils/rnnt_helper.py:119-142 get_workspace_size -> mi_transducer_workspace_bytes
+ *
+ * Conventions
+ *   - plain C: device pointers, sizes, a hipStream_t passed as void*; no torch types.
+ *   - every function returns 0 on success, 1 on an invalid value (mirrors RNNTStatus,
+ *     utils/global_constants.py:66-68), 2 if a HIP launch failed.  Nothing throws.
+ *   - all work is enqueued on `stream`; no call blocks the host, allocates or frees.
+ *   - all device memory is caller-owned.  `workspace` is scratch of at least
+ *     mi_transducer_workspace_bytes() bytes, 256-byte aligned; its contents after a
+ *     forward call are what the matching backward call reads, so keep it until then.
+ *     Concurrent calls must use different workspaces.
+ *   - acts:   [B,T,U,V(+D)] row-major contiguous raw LOGITS (the library normalises),
+ *             dtype code 0 = float32, 1 = bfloat16, 2 = float16; accumulation is fp32/fp64.
+ *   - labels: int64 [B,U-1]; act_lens, label_lens: int64 [B]; all on the device.
+ *     Lengths are clamped to [1,T] / [0,U-1] and label ids to [0,V-1] inside the
+ *     kernels so that a bad value can never address outside the tensors.
+ *   - limits: U <= 1024 (as the reference: one thread per label position,
+ *     utils/cuda_utils/gpu_rnnt.py:164), D <= 16, durations strictly ascending,
+ *     non-negative and holding 1 at position 0 or 1
+ *     (utils/cuda_utils/gpu_rnnt_kernel.py:1137-1148).
+ */
+#ifndef MI_TRANSDUCER_H_
+#define MI_TRANSDUCER_H_
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define MI_TRANSDUCER_SUCCESS 0
+#define MI_TRANSDUCER_INVALID_VALUE 1
+#define MI_TRANSDUCER_LAUNCH_FAILURE 2
+
+#define MI_DTYPE_F32 0
+#define MI_DTYPE_BF16 1
+#define MI_DTYPE_F16 2
+
+#define MI_TRANSDUCER_MAX_U 1024
+#define MI_TRANSDUCER_MAX_DURATIONS 16
+
+/* Library/ABI version; bumped whenever a signature below changes. */
+int mi_transducer_abi_version(void);
+
+/* Scratch bytes needed for a [B,T,U] lattice with D duration outputs (D = 0 for RNNT).
+ * Replaces get_workspace_size (utils/rnnt_helper.py:119-142); any dimension <= 0 is
+ * an invalid value, as there. */
+int mi_transducer_workspace_bytes(int B, int T, int U, int D, size_t* out_bytes);
+
+/* RNNT forward: log-softmax denominators of the valid cells (replaces reduce_max +
+ * reduce_exp, utils/cuda_utils/reduce.py:121-248), forward variables and
+ * costs[b] = -ll[b] * float32(1 + fastemit_lambda) (compute_alphas_kernel,
+ * utils/cuda_utils/gpu_rnnt_kernel.py:73-172; compute_costs_data,
+ * utils/rnnt_helper.py:106-116).  with_betas != 0 also runs the backward variables
+ * (compute_betas_kernel, gpu_rnnt_kernel.py:175-269), which mi_rnnt_backward needs;
+ * with_betas == 0 is the reference's score_forward (gpu_rnnt.py:250-265). */
+int mi_rnnt_forward(const void* acts, int act_dtype, const int64_t* labels, const int64_t* act_lens,
+                    const int64_t* label_lens, float* costs, int B, int T, int U, int V, int blank,
+                    float fastemit_lambda, int with_betas, void* workspace, size_t workspace_bytes, void* stream);
+
+/* RNNT backward: writes every element of grads[B,T,U,V] (same dtype as acts): the
+ * gradient of costs[b] w.r.t. the logits for valid cells, FastEmit and clamp folded
+ * in (compute_grad_kernel, gpu_rnnt_kernel.py:272-407), zeros for padded cells
+ * (replaces zeros_like + `grads *= 0`, rnnt_pytorch.py:58, gpu_rnnt.py:156).
+ * grad_scale (nullable, float32 [B]) multiplies utterance b's gradient after the
+ * clamp: it folds the autograd backward `grads.mul_(grad_output)` (rnnt_pytorch.py:88-92)
+ * and the 'mean' reduction's 1/B (rnnt_pytorch.py:77-81) into the same pass.
+ * Must follow mi_rnnt_forward(with_betas != 0) on the same workspace and inputs. */
+int mi_rnnt_backward(const void* acts, int act_dtype, const int64_t* labels, const int64_t* act_lens,
+                     const int64_t* label_lens, void* grads, const float* grad_scale, int B, int T, int U, int V,
+                     int blank, float fastemit_lambda, float clamp, void* workspace, size_t workspace_bytes,
+                     void* stream);
+
+/* rnnt_loss_gpu in one call (rnnt.py:138-236 -> GPURNNT.cost_and_grad / score_forward,
+ * gpu_rnnt.py:125-265): grads == NULL means forward only. */
+int mi_rnnt_loss(const void* acts, int act_dtype, const int64_t* labels, const int64_t* act_lens,
+                 const int64_t* label_lens, float* costs, void* grads, const float* grad_scale, int B, int T, int U,
+                 int V, int blank, float fastemit_lambda, float clamp, void* workspace, size_t workspace_bytes,
+                 void* stream);
+
+/* TDT.  acts is the COMBINED tensor [B,T,U,V+D]: V token logits (blank included)
+ * followed by D duration logits, exactly what TDTLossNumba.forward receives
+ * (rnnt_pytorch.py:554-583); the split, the .contiguous() copies and the duration
+ * log_softmax it performs are done inside the kernels.  durations_host: D ints in
+ * HOST memory.  Kernels replaced: compute_tdt_alphas_kernel / _betas_kernel /
+ * _grad_kernel (gpu_rnnt_kernel.py:888-1439) with sigma as there.  The gradient is
+ * w.r.t. the combined LOGITS: the duration block already carries the log-softmax
+ * Jacobian that torch autograd applies for the reference.
+ * use_plain_rnnt != 0 is the reference's omega branch (gpu_rnnt.py:606-682): the
+ * caller samples r < omega on the host; token logits then go through the plain RNNT
+ * kernels and the duration block of the gradient is zero. */
+int mi_tdt_forward(const void* acts, int act_dtype, const int64_t* labels, const int64_t* act_lens,
+                   const int64_t* label_lens, float* costs, int B, int T, int U, int V, int D,
+                   const int32_t* durations_host, int blank, float fastemit_lambda, float sigma, int use_plain_rnnt,
+                   int with_betas, void* workspace, size_t workspace_bytes, void* stream);
+
+int mi_tdt_backward(const void* acts, int act_dtype, const int64_t* labels, const int64_t* act_lens,
+                    const int64_t* label_lens, void* grads, const float* grad_scale, int B, int T, int U, int V, int D,
+                    const int32_t* durations_host, int blank, float fastemit_lambda, float clamp, float sigma,
+                    int use_plain_rnnt, void* workspace, size_t workspace_bytes, void* stream);
+
+int mi_tdt_loss(const void* acts, int act_dtype, const int64_t* labels, const int64_t* act_lens,
+                const int64_t* label_lens, float* costs, void* grads, const float* grad_scale, int B, int T, int U,
+                int V, int D, const int32_t* durations_host, int blank, float fastemit_lambda, float clamp, float sigma,
+                int use_plain_rnnt, void* workspace, size_t workspace_bytes, void* stream);
+
+/* Stage-level read-out for kernel parity tests (the reference tests launch each
+ * kernel on its own, tests/collections/asr/numba/rnnt_loss/utils/test_gpu_rnnt_kernel.py):
+ * copies what the last forward call left in `workspace` into plain [B,T,U] float32
+ * arrays (cells outside an utterance's lattice are set to 0) and [B] log-likelihoods.
+ * Any output pointer may be NULL.  betas / ll_backward are only meaningful after a
+ * forward call with with_betas != 0. */
+int mi_transducer_export_lattice(const void* workspace, size_t workspace_bytes, const int64_t* act_lens,
+                                 const int64_t* label_lens, int B, int T, int U, int D, float* denom, float* alphas,
+                                 float* betas, float* ll_forward, float* ll_backward, void* stream);
+
+/* out[0] = max(act_lens), out[1] = max(label_lens) (device int64[2]).  The host reads them
+ * back for the shape check of certify_inputs (rnnt_pytorch.py:628-634: T == max(act_lens),
+ * U == max(label_lens) + 1), which the reference does with two torch.max calls. */
+int mi_transducer_length_maxima(const int64_t* act_lens, const int64_t* label_lens, int B, int64_t* out,
+                                void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* MI_TRANSDUCER_H_ */

@@ -1,0 +1,113 @@
+"""ctypes binding of libmi_transducer.so (the HIP kernels behind a plain C ABI).
+
+The library is built in-tree by `build()` (hipcc, gfx950) and loaded from
+speech_amd/csrc/.  There is no fallback: if the library cannot be loaded, every
+entry point raises, so a silent non-HIP path cannot exist.
+"""
+
+import ctypes
+import os
+import subprocess
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+CSRC_DIR = os.path.join(_HERE, "csrc")
+INCLUDE_DIR = os.path.join(os.path.dirname(_HERE), "include")
+LIB_PATH = os.path.join(CSRC_DIR, "libmi_transducer.so")
+SOURCES = [os.path.join(CSRC_DIR, "mi_transducer.hip")]
+
+ABI_VERSION = 1
+SUCCESS, INVALID_VALUE, LAUNCH_FAILURE = 0, 1, 2
+DTYPE_F32, DTYPE_BF16, DTYPE_F16 = 0, 1, 2
+
+HIPCC_FLAGS = [
+    "--offload-arch=gfx950",
+    "-O3",
+    "-std=c++17",
+    "-fPIC",
+    "-shared",
+    # keep the compiler from forming packed-fp32 instructions
+    "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+]  # fmt: skip
+
+
+def build(verbose=False):
+    """Compile the HIP sources into speech_amd/csrc/libmi_transducer.so (cross-compiles without a GPU)."""
+    hipcc = os.environ.get("HIPCC", "hipcc")
+    cmd = [hipcc, *HIPCC_FLAGS, "-I", INCLUDE_DIR, "-o", LIB_PATH, *SOURCES]
+    proc = subprocess.run(cmd, capture_output=True, text=True)
+    if verbose or proc.returncode != 0:
+        print(" ".join(cmd))
+        print(proc.stdout)
+        print(proc.stderr)
+    if proc.returncode != 0:
+        raise RuntimeError("hipcc failed building libmi_transducer.so:\n" + proc.stderr)
+    global _lib
+    _lib = None
+    return LIB_PATH
+
+
+_lib = None
+
+_c_int, _c_float, _c_size_t, _vp = ctypes.c_int, ctypes.c_float, ctypes.c_size_t, ctypes.c_void_p
+
+# name -> argtypes, in the order of include/mi_transducer.h
+_SIGNATURES = {
+    "mi_transducer_abi_version": [],
+    "mi_transducer_workspace_bytes": [_c_int, _c_int, _c_int, _c_int, ctypes.POINTER(_c_size_t)],
+    "mi_rnnt_forward": [_vp, _c_int, _vp, _vp, _vp, _vp, _c_int, _c_int, _c_int, _c_int, _c_int, _c_float, _c_int,
+                        _vp, _c_size_t, _vp],
+    "mi_rnnt_backward": [_vp, _c_int, _vp, _vp, _vp, _vp, _vp, _c_int, _c_int, _c_int, _c_int, _c_int, _c_float,
+                         _c_float, _vp, _c_size_t, _vp],
+    "mi_rnnt_loss": [_vp, _c_int, _vp, _vp, _vp, _vp, _vp, _vp, _c_int, _c_int, _c_int, _c_int, _c_int, _c_float,
+                     _c_float, _vp, _c_size_t, _vp],
+    "mi_tdt_forward": [_vp, _c_int, _vp, _vp, _vp, _vp, _c_int, _c_int, _c_int, _c_int, _c_int, _vp, _c_int, _c_float,
+                       _c_float, _c_int, _c_int, _vp, _c_size_t, _vp],
+    "mi_tdt_backward": [_vp, _c_int, _vp, _vp, _vp, _vp, _vp, _c_int, _c_int, _c_int, _c_int, _c_int, _vp, _c_int,
+                        _c_float, _c_float, _c_float, _c_int, _vp, _c_size_t, _vp],
+    "mi_tdt_loss": [_vp, _c_int, _vp, _vp, _vp, _vp, _vp, _vp, _c_int, _c_int, _c_int, _c_int, _c_int, _vp, _c_int,
+                    _c_float, _c_float, _c_float, _c_int, _vp, _c_size_t, _vp],
+    "mi_transducer_export_lattice": [_vp, _c_size_t, _vp, _vp, _c_int, _c_int, _c_int, _c_int, _vp, _vp, _vp, _vp,
+                                     _vp, _vp],
+    "mi_transducer_length_maxima": [_vp, _vp, _c_int, _vp, _vp],
+}  # fmt: skip
+
+EXPORTED_SYMBOLS = tuple(_SIGNATURES)
+
+
+def lib():
+    """The loaded library; raises if it is missing or of another ABI version."""
+    global _lib
+    if _lib is None:
+        if not os.path.exists(LIB_PATH):
+            raise RuntimeError(
+                f"{LIB_PATH} is missing: the HIP extension has not been built "
+                "(run `python -c 'import __graft_entry__ as g; g.build()'`); there is no fallback path"
+            )
+        handle = ctypes.CDLL(LIB_PATH)
+        for name, argtypes in _SIGNATURES.items():
+            fn = getattr(handle, name)
+            fn.argtypes = argtypes
+            fn.restype = _c_int
+        got = handle.mi_transducer_abi_version()
+        if got != ABI_VERSION:
+            raise RuntimeError(f"libmi_transducer.so has ABI version {got}, expected {ABI_VERSION}: rebuild it")
+        _lib = handle
+    return _lib
+
+
+def check_status(status, what):
+    """Map the library's status codes to the reference's exception (rnnt.py:184-185, 219-234)."""
+    if status == SUCCESS:
+        return
+    if status == INVALID_VALUE:
+        raise RuntimeError(f"{what}: invalid value passed to the transducer-loss library")
+    raise RuntimeError(f"{what}: HIP kernel launch failed (status {status})")
+
+
+def workspace_bytes(B, T, U, D=0):
+    out = _c_size_t(0)
+    status = lib().mi_transducer_workspace_bytes(B, T, U, D, ctypes.byref(out))
+    if status != SUCCESS:
+        # rnnt.py:184-185
+        raise RuntimeError("Invalid parameter passed when calculating working space memory")
+    return int(out.value)

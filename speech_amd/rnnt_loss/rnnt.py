@@ -1,0 +1,203 @@
+"""Function-level seam of the transducer loss on MI355X.
+
+Mirrors nemo/collections/asr/parts/numba/rnnt_loss/rnnt.py: `rnnt_loss_gpu`
+(:138-236) and `tdt_loss_gpu` (:239-363) fill caller-owned `costs` / `grads`
+in place and return True; a non-success status becomes RuntimeError.  Below
+them the work is done by libmi_transducer.so on torch's current stream.  The
+split `*_forward` / `*_backward` functions are what the autograd Functions in
+rnnt_pytorch.py use: the gradient is produced in backward with grad_output
+folded in, instead of being stored in forward and rescaled later.
+
+Differences a caller can see:
+  * nothing blocks the host (the reference ends with stream.synchronize(),
+    utils/cuda_utils/gpu_rnnt.py:229);
+  * `tdt_loss_gpu` takes the combined [B,T,U,V+D] logits and returns the
+    gradient w.r.t. them (the kernels do the split and the duration
+    log-softmax that TDTLossNumba.forward does with torch ops, rnnt_pytorch.py:564-568);
+  * there is no CPU implementation here: CPU tensors raise.
+"""
+
+import ctypes
+
+import torch
+
+from speech_amd import _native
+
+_DTYPE_CODE = {
+    torch.float32: _native.DTYPE_F32,
+    torch.bfloat16: _native.DTYPE_BF16,
+    torch.float16: _native.DTYPE_F16,
+}
+
+
+def _dtype_code(t):
+    try:
+        return _DTYPE_CODE[t.dtype]
+    except KeyError:
+        raise TypeError(f"acts must be float32, bfloat16 or float16, got {t.dtype}") from None
+
+
+def _require_gpu(t, what):
+    if not t.is_cuda:
+        raise RuntimeError(f"{what}: this build runs on the GPU only; got a tensor on {t.device}")
+
+
+def _ptr(t):
+    return None if t is None else ctypes.c_void_p(t.data_ptr())
+
+
+def _stream(device):
+    return ctypes.c_void_p(torch.cuda.current_stream(device).cuda_stream)
+
+
+def _labels_ptr(labels):
+    # an empty [B,0] label matrix (U == 1) has no storage to point at
+    return _ptr(labels) if labels.numel() > 0 else None
+
+
+def _durations_array(durations):
+    arr = (ctypes.c_int32 * len(durations))(*[int(d) for d in durations])
+    return arr, ctypes.cast(arr, ctypes.c_void_p)
+
+
+def new_workspace(acts, num_durations=0):
+    """Scratch for one call (replaces torch.zeros(get_workspace_size(...)), rnnt.py:182-189; not zero-filled)."""
+    B, T, U = acts.shape[:3]
+    nbytes = _native.workspace_bytes(B, T, U, num_durations)
+    return torch.empty(nbytes, dtype=torch.uint8, device=acts.device)
+
+
+def length_maxima(act_lens, label_lens):
+    """Device int64[2] = (max(act_lens), max(label_lens)), enqueued on the current stream."""
+    _require_gpu(act_lens, "length_maxima")
+    out = torch.empty(2, dtype=torch.int64, device=act_lens.device)
+    with torch.cuda.device(act_lens.device):
+        status = _native.lib().mi_transducer_length_maxima(
+            _ptr(act_lens), _ptr(label_lens), act_lens.shape[0], _ptr(out), _stream(act_lens.device)
+        )
+    _native.check_status(status, "length_maxima")
+    return out
+
+
+def rnnt_forward(acts, labels, act_lens, label_lens, costs, blank, fastemit_lambda, with_betas, workspace):
+    _require_gpu(acts, "rnnt_forward")
+    B, T, U, V = acts.shape
+    with torch.cuda.device(acts.device):
+        status = _native.lib().mi_rnnt_forward(
+            _ptr(acts), _dtype_code(acts), _labels_ptr(labels), _ptr(act_lens), _ptr(label_lens), _ptr(costs),
+            B, T, U, V, int(blank), float(fastemit_lambda), int(bool(with_betas)),
+            _ptr(workspace), workspace.numel(), _stream(acts.device),
+        )  # fmt: skip
+    _native.check_status(status, "Could not calculate forward scores")
+
+
+def rnnt_backward(
+    acts, labels, act_lens, label_lens, grads, grad_scale, blank, fastemit_lambda, clamp, workspace
+):
+    _require_gpu(acts, "rnnt_backward")
+    B, T, U, V = acts.shape
+    with torch.cuda.device(acts.device):
+        status = _native.lib().mi_rnnt_backward(
+            _ptr(acts), _dtype_code(acts), _labels_ptr(labels), _ptr(act_lens), _ptr(label_lens), _ptr(grads),
+            _ptr(grad_scale), B, T, U, V, int(blank), float(fastemit_lambda), float(clamp),
+            _ptr(workspace), workspace.numel(), _stream(acts.device),
+        )  # fmt: skip
+    _native.check_status(status, "Could not calculate gradients")
+
+
+def tdt_forward(
+    acts, labels, act_lens, label_lens, costs, blank, durations, fastemit_lambda, sigma, use_plain_rnnt, with_betas,
+    workspace,
+):  # fmt: skip
+    _require_gpu(acts, "tdt_forward")
+    B, T, U, VD = acts.shape
+    D = len(durations)
+    keep, dur_ptr = _durations_array(durations)
+    with torch.cuda.device(acts.device):
+        status = _native.lib().mi_tdt_forward(
+            _ptr(acts), _dtype_code(acts), _labels_ptr(labels), _ptr(act_lens), _ptr(label_lens), _ptr(costs),
+            B, T, U, VD - D, D, dur_ptr, int(blank), float(fastemit_lambda), float(sigma), int(bool(use_plain_rnnt)),
+            int(bool(with_betas)), _ptr(workspace), workspace.numel(), _stream(acts.device),
+        )  # fmt: skip
+    del keep
+    _native.check_status(status, "Could not calculate forward scores")
+
+
+def tdt_backward(
+    acts, labels, act_lens, label_lens, grads, grad_scale, blank, durations, fastemit_lambda, clamp, sigma,
+    use_plain_rnnt, workspace,
+):  # fmt: skip
+    _require_gpu(acts, "tdt_backward")
+    B, T, U, VD = acts.shape
+    D = len(durations)
+    keep, dur_ptr = _durations_array(durations)
+    with torch.cuda.device(acts.device):
+        status = _native.lib().mi_tdt_backward(
+            _ptr(acts), _dtype_code(acts), _labels_ptr(labels), _ptr(act_lens), _ptr(label_lens), _ptr(grads),
+            _ptr(grad_scale), B, T, U, VD - D, D, dur_ptr, int(blank), float(fastemit_lambda), float(clamp),
+            float(sigma), int(bool(use_plain_rnnt)), _ptr(workspace), workspace.numel(), _stream(acts.device),
+        )  # fmt: skip
+    del keep
+    _native.check_status(status, "Could not calculate gradients")
+
+
+def export_lattice(workspace, act_lens, label_lens, B, T, U, num_durations=0):
+    """(denom, alphas, betas, ll_forward, ll_backward) as plain float32 tensors, for stage-level checks."""
+    dev = workspace.device
+    denom = torch.empty(B, T, U, dtype=torch.float32, device=dev)
+    alphas = torch.empty_like(denom)
+    betas = torch.empty_like(denom)
+    llf = torch.empty(B, dtype=torch.float32, device=dev)
+    llb = torch.empty_like(llf)
+    with torch.cuda.device(dev):
+        status = _native.lib().mi_transducer_export_lattice(
+            _ptr(workspace), workspace.numel(), _ptr(act_lens), _ptr(label_lens), B, T, U, num_durations,
+            _ptr(denom), _ptr(alphas), _ptr(betas), _ptr(llf), _ptr(llb), _stream(dev),
+        )  # fmt: skip
+    _native.check_status(status, "export_lattice")
+    return denom, alphas, betas, llf, llb
+
+
+def rnnt_loss_gpu(
+    acts, labels, input_lengths, label_lengths, costs, grads, blank_label, fastemit_lambda, clamp, num_threads=0
+):
+    """Drop-in for rnnt.py:138-236: costs (float32 [B]) and grads (or None) are filled in place."""
+    del num_threads  # an OpenMP knob of the reference's CPU path; unused on the GPU there too
+    _require_gpu(acts, "rnnt_loss_gpu")
+    B, T, U, V = acts.shape
+    workspace = new_workspace(acts)  # raises the reference's RuntimeError for non-positive dims
+    if costs.dtype != torch.float32:
+        raise TypeError("costs must be float32")
+    with torch.cuda.device(acts.device):
+        status = _native.lib().mi_rnnt_loss(
+            _ptr(acts), _dtype_code(acts), _labels_ptr(labels), _ptr(input_lengths), _ptr(label_lengths), _ptr(costs),
+            _ptr(grads), None, B, T, U, V, int(blank_label), float(fastemit_lambda), float(clamp),
+            _ptr(workspace), workspace.numel(), _stream(acts.device),
+        )  # fmt: skip
+    _native.check_status(status, "Could not calculate forward scores")
+    # the caching allocator frees `workspace` in stream order, so it may go out of scope here
+    return True
+
+
+def tdt_loss_gpu(
+    acts, labels, input_lengths, label_lengths, costs, grads, blank_label, durations, fastemit_lambda, clamp,
+    num_threads=0, sigma=0.0, use_plain_rnnt=False,
+):  # fmt: skip
+    """TDT counterpart (rnnt.py:239-363) on the combined [B,T,U,V+D] logits; costs is float32 [B]."""
+    del num_threads
+    _require_gpu(acts, "tdt_loss_gpu")
+    B, T, U, VD = acts.shape
+    D = len(durations)
+    workspace = new_workspace(acts, D)
+    if costs.dtype != torch.float32:
+        raise TypeError("costs must be float32")
+    keep, dur_ptr = _durations_array(durations)
+    with torch.cuda.device(acts.device):
+        status = _native.lib().mi_tdt_loss(
+            _ptr(acts), _dtype_code(acts), _labels_ptr(labels), _ptr(input_lengths), _ptr(label_lengths), _ptr(costs),
+            _ptr(grads), None, B, T, U, VD - D, D, dur_ptr, int(blank_label), float(fastemit_lambda), float(clamp),
+            float(sigma), int(bool(use_plain_rnnt)), _ptr(workspace), workspace.numel(), _stream(acts.device),
+        )  # fmt: skip
+    del keep
+    _native.check_status(status, "Could not calculate forward scores")
+    return True

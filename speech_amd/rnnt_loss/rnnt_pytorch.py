@@ -1,0 +1,308 @@
+"""Module-level call surface of the transducer loss on MI355X.
+
+Keeps the interface of nemo/collections/asr/parts/numba/rnnt_loss/rnnt_pytorch.py:
+`RNNTLossNumba` (:392-439) and `TDTLossNumba` (:513-583) with the same
+constructor arguments, the same `forward(acts, labels, act_lens, label_lens)`
+(names and order are part of the contract: the outer wrapper calls by keyword,
+nemo/collections/asr/losses/rnnt.py:484-491), the same mutable attributes
+(`blank`, `reduction`, `fastemit_lambda`, `clamp`, `durations`, `sigma`, `omega`),
+the same input validation and exceptions (`certify_inputs`, :601-634) and the
+same outputs: float32 costs of shape [B] (reduction None/'none') or [1]
+('sum'/'mean'), gradient only w.r.t. `acts`.
+
+What is done differently underneath:
+  * `acts` are raw logits of dtype float32, bfloat16 or float16 on the GPU; the
+    log-softmax happens inside the kernels.  CPU tensors raise (no CPU path here).
+  * the gradient is computed in `backward`, by one kernel pass that already folds
+    in `grad_output`, the 'mean' reduction's 1/B, FastEmit and the clamp; forward
+    keeps a few MB of lattice state instead of a gradient tensor the size of `acts`.
+  * the shape-vs-lengths check reads both maxima back with one small copy that
+    overlaps the forward kernels instead of two blocking torch.max calls.
+"""
+
+import random
+
+import torch
+from torch.autograd import Function
+from torch.nn import Module
+
+from speech_amd.rnnt_loss import rnnt
+
+__all__ = ['RNNTLossNumba', 'TDTLossNumba', 'RNNTLossMI355X', 'TDTLossMI355X', 'certify_inputs']
+
+
+def check_type(var, t, name):
+    if var.dtype is not t:
+        raise TypeError("{} must be {}".format(name, t))
+
+
+def check_contiguous(var, name):
+    if not var.is_contiguous():
+        raise ValueError("{} must be contiguous".format(name))
+
+
+def check_dim(var, dim, name):
+    if len(var.shape) != dim:
+        raise ValueError("{} must be {}D".format(name, dim))
+
+
+class _PendingLengthCheck:
+    """The T == max(act_lens), U == max(label_lens)+1 test of certify_inputs, split in two
+    so that the read-back of the maxima overlaps kernels enqueued in between."""
+
+    def __init__(self, log_probs, lengths, label_lengths):
+        self.T, self.U = log_probs.shape[1:3]
+        if lengths.is_cuda:
+            maxima = rnnt.length_maxima(lengths, label_lengths)
+            self.host = torch.empty(2, dtype=torch.int64, pin_memory=True)
+            self.host.copy_(maxima, non_blocking=True)
+            self.event = torch.cuda.Event()
+            self.event.record(torch.cuda.current_stream(lengths.device))
+        else:
+            self.host = torch.stack([torch.max(lengths), torch.max(label_lengths)])
+            self.event = None
+
+    def finish(self):
+        if self.event is not None:
+            self.event.synchronize()
+        max_T, max_U = int(self.host[0]), int(self.host[1])
+        if self.T != max_T:
+            raise ValueError(f"Input length mismatch! Given T: {self.T}, Expected max T from input lengths: {max_T}")
+        if self.U != max_U + 1:
+            raise ValueError(
+                f"Output length mismatch! Given U: {self.U}, Expected max U from target lengths: {max_U} + 1"
+            )
+
+
+def _certify_static(log_probs, labels, lengths, label_lengths):
+    check_type(labels, torch.int64, "labels")
+    check_type(label_lengths, torch.int64, "label_lengths")
+    check_type(lengths, torch.int64, "lengths")
+    check_contiguous(log_probs, "log_probs")
+    check_contiguous(labels, "labels")
+    check_contiguous(label_lengths, "label_lengths")
+    check_contiguous(lengths, "lengths")
+
+    if lengths.shape[0] != log_probs.shape[0]:
+        raise ValueError(
+            f"Must have a length per example. "
+            f"Given lengths dim: {lengths.shape[0]}, "
+            f"Log probs dim : {log_probs.shape[0]}"
+        )
+    if label_lengths.shape[0] != log_probs.shape[0]:
+        raise ValueError(
+            "Must have a label length per example. "
+            f"Given label lengths dim : {label_lengths.shape[0]}, "
+            f"Log probs dim : {log_probs.shape[0]}"
+        )
+
+    check_dim(log_probs, 4, "log_probs")
+    check_dim(labels, 2, "labels")
+    check_dim(lengths, 1, "lenghts")
+    check_dim(label_lengths, 1, "label_lenghts")
+
+
+def certify_inputs(log_probs, labels, lengths, label_lengths):
+    """Same checks, order, exception types and messages as rnnt_pytorch.py:601-634."""
+    _certify_static(log_probs, labels, lengths, label_lengths)
+    _PendingLengthCheck(log_probs, lengths, label_lengths).finish()
+
+
+def _check_same_device(acts, *others):
+    for t in others:
+        if t.device != acts.device:
+            raise ValueError(f"labels and lengths must be on the device of acts ({acts.device}), got {t.device}")
+
+
+def _reduce_costs(costs, reduction, batch):
+    # rnnt_pytorch.py:75-81: 'sum' and 'mean' give shape [1]; anything else is per utterance
+    if reduction in ['sum', 'mean']:
+        costs = costs.sum().unsqueeze_(-1)
+        if reduction == 'mean':
+            costs /= batch
+    return costs
+
+
+def _grad_scale(grad_output, reduction, batch, device):
+    # what the reference applies to its stored gradient: /B for 'mean' in forward
+    # (rnnt_pytorch.py:77-81), then * grad_output broadcast over the batch in backward (:88-92)
+    scale = grad_output.detach().to(device=device, dtype=torch.float32).reshape(-1)
+    if scale.numel() == 1:
+        scale = scale.expand(batch)
+    elif scale.numel() != batch:
+        raise RuntimeError(f"grad_output has {scale.numel()} elements, expected 1 or {batch}")
+    if reduction == 'mean':
+        scale = scale / batch
+    return scale.contiguous()
+
+
+class _RNNTNumba(Function):
+    @staticmethod
+    def forward(ctx, acts, labels, act_lens, label_lens, blank, reduction, fastemit_lambda, clamp):
+        _certify_static(acts, labels, act_lens, label_lens)
+        if clamp < 0:
+            raise ValueError("`clamp` must be 0.0 or positive float value.")
+        if not acts.is_cuda:
+            raise RuntimeError(
+                "RNNTLossNumba (MI355X build) has no CPU implementation: move acts, labels and lengths to the GPU"
+            )
+        _check_same_device(acts, labels, act_lens, label_lens)
+        pending = _PendingLengthCheck(acts, act_lens, label_lens)
+
+        need_grad = ctx.needs_input_grad[0]
+        batch = acts.size(0)
+        costs = torch.empty(batch, device=acts.device, dtype=torch.float32)
+        workspace = rnnt.new_workspace(acts)
+        rnnt.rnnt_forward(acts, labels, act_lens, label_lens, costs, blank, fastemit_lambda, need_grad, workspace)
+        pending.finish()  # raises ValueError exactly where certify_inputs would
+
+        costs = _reduce_costs(costs, reduction, batch)
+        if need_grad:
+            ctx.save_for_backward(acts, labels, act_lens, label_lens, workspace)
+            ctx.params = (blank, reduction, fastemit_lambda, clamp)
+        return costs
+
+    @staticmethod
+    def backward(ctx, grad_output):
+        acts, labels, act_lens, label_lens, workspace = ctx.saved_tensors
+        blank, reduction, fastemit_lambda, clamp = ctx.params
+        grads = torch.empty_like(acts)
+        scale = _grad_scale(grad_output, reduction, acts.size(0), acts.device)
+        rnnt.rnnt_backward(acts, labels, act_lens, label_lens, grads, scale, blank, fastemit_lambda, clamp, workspace)
+        return grads, None, None, None, None, None, None, None
+
+
+class _TDTNumba(Function):
+    """Token-and-Duration Transducer loss (arXiv:2304.06795) on the combined logits."""
+
+    @staticmethod
+    def forward(
+        ctx, acts, labels, act_lens, label_lens, blank, durations, reduction, fastemit_lambda, clamp, sigma, omega
+    ):
+        _certify_static(acts, labels, act_lens, label_lens)
+        if clamp < 0:
+            raise ValueError("`clamp` must be 0.0 or positive float value.")
+        if not acts.is_cuda:
+            # rnnt_pytorch.py:137-140
+            raise ValueError("TDT is not yet implemented for non CUDA computation.")
+        _check_same_device(acts, labels, act_lens, label_lens)
+        durations = [int(d) for d in durations]
+        if acts.shape[-1] <= len(durations):
+            raise ValueError("acts must hold the token logits followed by one logit per duration")
+        pending = _PendingLengthCheck(acts, act_lens, label_lens)
+
+        need_grad = ctx.needs_input_grad[0]
+        batch = acts.size(0)
+        costs = torch.empty(batch, device=acts.device, dtype=torch.float32)
+        workspace = rnnt.new_workspace(acts, len(durations))
+        # gpu_rnnt.py:606-607: one host-side draw per call decides between the TDT and the plain RNNT kernels
+        use_plain_rnnt = random.uniform(0, 1) < omega
+        rnnt.tdt_forward(
+            acts, labels, act_lens, label_lens, costs, blank, durations, fastemit_lambda, sigma, use_plain_rnnt,
+            need_grad, workspace,
+        )  # fmt: skip
+        pending.finish()
+
+        # the reference allocates TDT costs in the dtype of acts (rnnt_pytorch.py:145)
+        costs = _reduce_costs(costs, reduction, batch).to(acts.dtype)
+        if need_grad:
+            ctx.save_for_backward(acts, labels, act_lens, label_lens, workspace)
+            ctx.params = (blank, durations, reduction, fastemit_lambda, clamp, sigma, use_plain_rnnt)
+        return costs
+
+    @staticmethod
+    def backward(ctx, grad_output):
+        acts, labels, act_lens, label_lens, workspace = ctx.saved_tensors
+        blank, durations, reduction, fastemit_lambda, clamp, sigma, use_plain_rnnt = ctx.params
+        grads = torch.empty_like(acts)
+        scale = _grad_scale(grad_output, reduction, acts.size(0), acts.device)
+        rnnt.tdt_backward(
+            acts, labels, act_lens, label_lens, grads, scale, blank, durations, fastemit_lambda, clamp, sigma,
+            use_plain_rnnt, workspace,
+        )  # fmt: skip
+        return grads, None, None, None, None, None, None, None, None, None, None
+
+
+class RNNTLossNumba(Module):
+    """
+    Parameters:
+        blank (int, optional): blank label. Default: 0.
+        reduction (string, optional): 'none' | 'mean' | 'sum' (None behaves as 'none'). Default: 'mean'
+        fastemit_lambda: scaling factor of the FastEmit regularisation (arXiv:2010.11148).
+        clamp: when > 0, every gradient element is clamped to [-clamp, clamp]; <= 0 disables it.
+    """
+
+    def __init__(self, blank=0, reduction='mean', fastemit_lambda: float = 0.0, clamp: float = -1):
+        super().__init__()
+        self.blank = blank
+        self.fastemit_lambda = fastemit_lambda
+        self.clamp = float(clamp) if clamp > 0 else 0.0
+        self.reduction = reduction
+        self.loss = _RNNTNumba.apply
+
+    def forward(self, acts, labels, act_lens, label_lens):
+        """
+        acts: [B, T, U, V] logits from the joint network (blank included in V)
+        labels: [B, U-1] int64 targets, zero padded
+        act_lens: [B] int64 number of valid frames per utterance
+        label_lens: [B] int64 number of valid labels per utterance
+        """
+        return self.loss(
+            acts, labels, act_lens, label_lens, self.blank, self.reduction, self.fastemit_lambda, self.clamp
+        )
+
+
+class TDTLossNumba(Module):
+    """
+    Parameters:
+        blank (int): blank label (index within the token logits).
+        durations: durations of the TDT model, ascending, e.g. [0, 1, 2, 3, 4]; must hold 1 at position 0 or 1.
+        reduction, fastemit_lambda, clamp: as RNNTLossNumba.
+        sigma: logit under-normalisation constant (recommended 0.05).
+        omega: probability of using the plain RNNT loss for a call.
+    """
+
+    def __init__(
+        self,
+        blank,
+        durations=None,
+        reduction='mean',
+        fastemit_lambda: float = 0.0,
+        clamp: float = -1,
+        sigma: float = 0.0,
+        omega: float = 0.0,
+    ):
+        super().__init__()
+        self.blank = blank
+        self.durations = durations if durations is not None else []
+        self.fastemit_lambda = fastemit_lambda
+        self.clamp = float(clamp) if clamp > 0 else 0.0
+        self.reduction = reduction
+        self.loss = _TDTNumba.apply
+        self.sigma = sigma
+        self.omega = omega
+
+    def forward(self, acts, labels, act_lens, label_lens):
+        """
+        acts: [B, T, U, V + D] logits: V token logits (blank included) then D = len(durations) duration logits
+        labels, act_lens, label_lens: as RNNTLossNumba
+        """
+        return self.loss(
+            acts,
+            labels,
+            act_lens,
+            label_lens,
+            self.blank,
+            self.durations,
+            self.reduction,
+            self.fastemit_lambda,
+            self.clamp,
+            self.sigma,
+            self.omega,
+        )
+
+
+# names that say what they are; the *Numba names are kept so that code written
+# against the reference runs unchanged
+RNNTLossMI355X = RNNTLossNumba
+TDTLossMI355X = TDTLossNumba

@@ -1,0 +1,102 @@
+"""CPU-side checks: the C-ABI library loads and exports every declared symbol,
+the host-side validation mirrors the reference, and nothing in the package
+reaches for the oracle."""
+
+import os
+import re
+
+import pytest
+import torch
+
+from speech_amd import _native
+from speech_amd.rnnt_loss.rnnt_pytorch import RNNTLossNumba, TDTLossNumba, certify_inputs
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+@pytest.fixture(scope="module")
+def built_lib():
+    if not os.path.exists(_native.LIB_PATH):
+        _native.build()
+    return _native.lib()
+
+
+def test_library_exports_every_symbol_declared_in_the_header(built_lib):
+    header = open(os.path.join(ROOT, "include", "mi_transducer.h")).read()
+    declared = set(re.findall(r"^int (mi_[a-z_]+)\(", header, flags=re.M))
+    assert declared == set(_native.EXPORTED_SYMBOLS)
+    for name in declared:
+        assert hasattr(built_lib, name), name
+    assert built_lib.mi_transducer_abi_version() == _native.ABI_VERSION
+
+
+def test_workspace_size_and_invalid_dimensions(built_lib):
+    small = _native.workspace_bytes(1, 2, 3, 0)
+    big = _native.workspace_bytes(16, 375, 121, 0)
+    assert 0 < small < big
+    assert _native.workspace_bytes(16, 375, 121, 5) > big
+    # utils/rnnt_helper.py:119-142: any non-positive dimension is an invalid value -> RuntimeError (rnnt.py:184-185)
+    for dims in [(0, 2, 3, 0), (1, 0, 3, 0), (1, 2, 0, 0), (1, 2, 1025, 0), (1, 2, 3, 17)]:
+        with pytest.raises(RuntimeError):
+            _native.workspace_bytes(*dims)
+
+
+def test_null_and_bad_arguments_return_invalid_value_without_touching_the_gpu(built_lib):
+    # every check happens on the host before any HIP call
+    assert built_lib.mi_rnnt_forward(None, 0, None, None, None, None, 1, 2, 3, 4, 0, 0.0, 0, None, 0, None) == 1
+    assert built_lib.mi_tdt_forward(None, 0, None, None, None, None, 1, 2, 3, 4, 2, None, 0, 0.0, 0.0, 0, 0, None, 0, None) == 1
+    assert built_lib.mi_transducer_length_maxima(None, None, 1, None, None) == 1
+
+
+def test_constructor_attributes_match_the_reference_conventions():
+    loss = RNNTLossNumba()
+    assert (loss.blank, loss.reduction, loss.fastemit_lambda, loss.clamp) == (0, 'mean', 0.0, 0.0)
+    assert RNNTLossNumba(clamp=2).clamp == 2.0 and RNNTLossNumba(clamp=-1).clamp == 0.0
+    tdt = TDTLossNumba(blank=5)
+    assert tdt.durations == [] and tdt.sigma == 0.0 and tdt.omega == 0.0
+    loss.reduction = None  # the outer wrapper mutates these (nemo/collections/asr/losses/rnnt.py:484-491)
+    loss.blank = 3
+
+
+def test_certify_inputs_on_cpu_tensors():
+    acts = torch.zeros(2, 4, 3, 5)
+    labels = torch.ones(2, 2, dtype=torch.int64)
+    act_lens = torch.tensor([4, 3])
+    label_lens = torch.tensor([2, 1])
+    certify_inputs(acts, labels, act_lens, label_lens)
+    with pytest.raises(TypeError, match="labels must be"):
+        certify_inputs(acts, labels.int(), act_lens, label_lens)
+    with pytest.raises(TypeError, match="label_lengths must be"):
+        certify_inputs(acts, labels, act_lens, label_lens.int())
+    with pytest.raises(ValueError, match="log_probs must be contiguous"):
+        certify_inputs(acts.transpose(0, 1), labels, act_lens, label_lens)
+    with pytest.raises(ValueError, match="log_probs must be 4D"):
+        certify_inputs(acts[0], labels, act_lens[:1].repeat(4), label_lens[:1].repeat(4))
+    with pytest.raises(ValueError, match="Input length mismatch"):
+        certify_inputs(acts, labels, act_lens - 1, label_lens)
+    with pytest.raises(ValueError, match="Output length mismatch"):
+        certify_inputs(acts, labels, act_lens, label_lens - 1)
+
+
+def test_cpu_tensors_are_refused_loudly():
+    acts = torch.zeros(1, 2, 2, 3, requires_grad=True)
+    labels = torch.ones(1, 1, dtype=torch.int64)
+    with pytest.raises(RuntimeError, match="no CPU implementation"):
+        RNNTLossNumba()(acts, labels, torch.tensor([2]), torch.tensor([1]))
+    with pytest.raises(ValueError, match="non CUDA"):
+        TDTLossNumba(blank=0, durations=[0, 1])(acts, labels, torch.tensor([2]), torch.tensor([1]))
+
+
+def test_missing_library_fails_loudly(monkeypatch, tmp_path):
+    monkeypatch.setattr(_native, "LIB_PATH", str(tmp_path / "libmi_transducer.so"))
+    monkeypatch.setattr(_native, "_lib", None)
+    with pytest.raises(RuntimeError, match="no fallback"):
+        _native.lib()
+
+
+def test_package_never_imports_the_oracle():
+    for dirpath, _, files in os.walk(os.path.join(ROOT, "speech_amd")):
+        for name in files:
+            if name.endswith((".py", ".hip", ".h")):
+                text = open(os.path.join(dirpath, name)).read()
+                assert "oracle" not in text.lower(), os.path.join(dirpath, name)
