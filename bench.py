@@ -1,0 +1,198 @@
+#!/usr/bin/env python3
+"""Benchmark of the transducer-loss hot path on one MI355X.
+
+A step is one forward + backward of the loss module over one resident batch:
+    costs = loss(acts, labels, act_lens, label_lens); costs.sum().backward()
+on the north-star workload (RNNT, B=16, T=375, U+1=121, V=1025, fp32, variable
+lengths), inputs already in HBM.  Prints ONE JSON line:
+  value        logit elements per second (B*T*U*V / step time)
+  roofline     the gradient-stream kernel (the dominant one): algorithmic bytes per launch /
+               its mean duration, measured with HIP events around the launches of the timed steps
+  cpu_baseline the C restatement of the reference's CPU path on a bounded sample, host cores
+  kernels      mean duration of each pipeline kernel over the timed steps (ms)
+  copy_probe   bandwidth a plain device copy reaches on this GPU (GB/s, read + write)
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload 0..4] [--no-cpu-baseline]
+"""
+
+import argparse
+import ctypes
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBPS = 8000.0  # MI355X HBM3E, published peak
+
+# HBM bytes per launch of grad_stream_kernel from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of
+# this script, scaled by what the same counters read for mi_transducer_copy_probe of known size
+# (summaries under profiles/).  None = not measured for that workload.
+MEASURED_TRAFFIC_BYTES = {}
+
+
+def parse_args():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=30)
+    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--workload", type=int, default=1, help="index into speech_amd.synthetic.CONFIGS (1 = north star)")
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--cpu-sample-utterances", type=int, default=8)
+    return ap.parse_args()
+
+
+def cpu_baseline(cfg, acts, labels, act_lens, label_lens, n_utt):
+    """The reference's CPU path (log_softmax, per-utterance lattice, sparse gradient, softmax
+    Jacobian) restated in C, timed on the host cores over the first n_utt utterances."""
+    import numpy as np
+
+    import oracle
+
+    threads = max(1, min(16, os.cpu_count() or 1))
+    n_utt = min(n_utt, cfg.B)
+    x = acts[:n_utt].float().cpu().numpy()
+    lab = labels[:n_utt].cpu().numpy()
+    al = act_lens[:n_utt].cpu().numpy()
+    ll = label_lens[:n_utt].cpu().numpy()
+    lam, clamp = cfg.fastemit_lambda, max(cfg.clamp, 0.0)
+    t0 = time.perf_counter()
+    if cfg.D:
+        oracle.tdt_loss(x, lab, al, ll, cfg.blank, cfg.durations, cfg.sigma, lam, clamp, dtype=np.float32,
+                        num_threads=threads)  # fmt: skip
+    else:
+        oracle.rnnt_cpu_path(x, lab, al, ll, cfg.blank, lam, clamp, dtype=np.float32, num_threads=threads)
+    dt = time.perf_counter() - t0
+    return {
+        "value": x.size / dt,
+        "unit": "logit elems/s",
+        "cores": threads,
+        "kind": "port",
+        "sample": f"first {n_utt} of {cfg.B} utterances of the same batch, full T x U x V, one pass, {dt:.2f} s wall",
+    }
+
+
+def main():
+    args = parse_args()
+    if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
+        print("bench.py: this build measures one GPU only; run with --gpus 1 (the loss is data-parallel over "
+              "utterances, nothing is exchanged between GPUs)", file=sys.stderr)  # fmt: skip
+        sys.exit(2)
+
+    import torch
+
+    from speech_amd import RNNTLossNumba, TDTLossNumba, _native, synthetic
+
+    if not torch.cuda.is_available():
+        print("bench.py: no GPU visible", file=sys.stderr)
+        sys.exit(2)
+    dev = torch.device("cuda:0")
+    torch.cuda.set_device(dev)
+    _native.lib()  # fail now if the HIP library is missing
+
+    cfg, acts, labels, act_lens, label_lens = synthetic.make_inputs(args.workload, device=dev, generate_on_device=True)
+    acts.requires_grad_(True)
+    if cfg.D:
+        loss = TDTLossNumba(blank=cfg.blank, durations=cfg.durations, reduction='none',
+                            fastemit_lambda=cfg.fastemit_lambda, clamp=cfg.clamp, sigma=cfg.sigma)  # fmt: skip
+    else:
+        loss = RNNTLossNumba(blank=cfg.blank, reduction='none', fastemit_lambda=cfg.fastemit_lambda, clamp=cfg.clamp)
+    nbytes = synthetic.algorithmic_bytes(cfg, act_lens, label_lens)
+
+    def step():
+        acts.grad = None
+        costs = loss(acts, labels, act_lens, label_lens)
+        costs.sum().backward()
+        return costs
+
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+
+    _native.profile_enable(args.steps)
+    start_ev, stop_ev = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    start_ev.record()
+    for _ in range(args.steps):
+        costs = step()
+    stop_ev.record()
+    torch.cuda.synchronize()
+    wall = time.perf_counter() - t0
+    kernels = _native.profile_read()
+    _native.profile_disable()
+    ms_per_step = wall * 1e3 / args.steps
+    event_ms_per_step = start_ev.elapsed_time(stop_ev) / args.steps
+    assert os.environ.get("MI_BENCH_ALLOW_NONFINITE") or bool(torch.isfinite(costs).all()), "non-finite costs"
+
+    # copy yardstick: 1 GiB device-to-device
+    n = 1 << 30
+    src = torch.empty(n, dtype=torch.uint8, device=dev)
+    dst = torch.empty_like(src)
+    stream = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+    for _ in range(3):
+        _native.lib().mi_transducer_copy_probe(src.data_ptr(), dst.data_ptr(), n, stream)
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    e0.record()
+    for _ in range(10):
+        _native.lib().mi_transducer_copy_probe(src.data_ptr(), dst.data_ptr(), n, stream)
+    e1.record()
+    torch.cuda.synchronize()
+    copy_gbps = 2 * n * 10 / (e0.elapsed_time(e1) * 1e-3) / 1e9
+    del src, dst
+
+    grad_ms, grad_n = kernels["grad_stream_kernel"]
+    grad_avg_s = grad_ms * 1e-3 / max(grad_n, 1)
+    achieved = nbytes["grad_stream"] / grad_avg_s / 1e9
+    result = {
+        "metric": "RNNT/TDT loss fwd+bwd: logit elems/s and achieved HBM GB/s vs peak",
+        "value": cfg.elems / (ms_per_step * 1e-3),
+        "unit": "logit elems/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": ms_per_step,
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": {torch.float32: "f32", torch.bfloat16: "bf16", torch.float16: "f16"}[cfg.dtype],
+        "data": "synthetic",
+        "config": {
+            "workload": cfg.name,
+            "B": cfg.B, "T": cfg.T, "U": cfg.U, "V": cfg.V, "D": cfg.D,
+            "valid_cells": nbytes["c_valid"], "cells": nbytes["cells"],
+            "fastemit_lambda": cfg.fastemit_lambda, "clamp": cfg.clamp, "sigma": cfg.sigma,
+        },
+        "whole_job": {
+            "algorithmic_bytes": nbytes["total"],
+            "achieved_GBps": nbytes["total"] / (ms_per_step * 1e-3) / 1e9,
+            "frac_of_peak": nbytes["total"] / (ms_per_step * 1e-3) / 1e9 / HBM_PEAK_GBPS,
+            "event_ms_per_step": event_ms_per_step,
+        },
+        "roofline": {
+            "kernel": "grad_stream_kernel",
+            "bound": "hbm",
+            "achieved": achieved,
+            "peak": HBM_PEAK_GBPS,
+            "unit": "GB/s",
+            "frac": achieved / HBM_PEAK_GBPS,
+            "traffic": MEASURED_TRAFFIC_BYTES.get(cfg.name),
+            "algorithmic_bytes_per_launch": nbytes["grad_stream"],
+            "avg_launch_ms": grad_avg_s * 1e3,
+            "launches": grad_n,
+        },
+        "kernels": {k: (ms / max(n_, 1)) for k, (ms, n_) in kernels.items()},
+        "copy_probe_GBps": copy_gbps,
+    }  # fmt: skip
+    if not args.no_cpu_baseline:
+        result["cpu_baseline"] = cpu_baseline(
+            cfg, acts.detach(), labels, act_lens, label_lens, args.cpu_sample_utterances
+        )
+    print(json.dumps(result))
+
+
+if __name__ == "__main__":
+    main()

@@ -127,6 +127,27 @@ int mi_transducer_export_lattice(const void* workspace, size_t workspace_bytes, 
 int mi_transducer_length_maxima(const int64_t* act_lens, const int64_t* label_lens, int B, int64_t* out,
                                 void* stream);
 
+/* ---- benchmark aids (no counterpart in the reference) --------------------------------
+ * Per-kernel timing of the launches a harness itself makes: after
+ * mi_transducer_profile_enable(n), each of the next n launches of every pipeline kernel is
+ * bracketed by a pair of HIP events on its stream (enable creates the events: the one
+ * place this library allocates).  mi_transducer_profile_read waits for the recorded
+ * launches of one kernel class, returns their summed duration and count, and resets that
+ * class.  Not thread-safe; leave disabled outside benchmarks. */
+#define MI_PROFILE_DENOM 0   /* denom_gather_kernel */
+#define MI_PROFILE_LATTICE 1 /* rnnt_lattice_kernel / tdt_lattice_kernel */
+#define MI_PROFILE_CELL 2    /* rnnt_cell_kernel / tdt_cell_kernel */
+#define MI_PROFILE_GRAD 3    /* grad_stream_kernel */
+#define MI_PROFILE_KERNELS 4
+int mi_transducer_profile_enable(int max_launches);
+int mi_transducer_profile_read(int kernel_id, float* total_ms, int* launches);
+int mi_transducer_profile_disable(void);
+
+/* Plain device-to-device copy of `bytes` (multiple of 16, 16-byte aligned pointers) with a
+ * grid-stride 16-byte-per-lane kernel: the known-size yardstick for hardware traffic
+ * counters and for the copy bandwidth the GPU reaches in practice. */
+int mi_transducer_copy_probe(const void* src, void* dst, size_t bytes, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

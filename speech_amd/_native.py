@@ -12,7 +12,8 @@ import subprocess
 _HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC_DIR = os.path.join(_HERE, "csrc")
 INCLUDE_DIR = os.path.join(os.path.dirname(_HERE), "include")
-LIB_PATH = os.path.join(CSRC_DIR, "libmi_transducer.so")
+# MI_TRANSDUCER_LIB lets a kernel developer point at an experimental build of the same ABI
+LIB_PATH = os.environ.get("MI_TRANSDUCER_LIB") or os.path.join(CSRC_DIR, "libmi_transducer.so")
 SOURCES = [os.path.join(CSRC_DIR, "mi_transducer.hip")]
 
 ABI_VERSION = 1
@@ -69,6 +70,10 @@ _SIGNATURES = {
     "mi_transducer_export_lattice": [_vp, _c_size_t, _vp, _vp, _c_int, _c_int, _c_int, _c_int, _vp, _vp, _vp, _vp,
                                      _vp, _vp],
     "mi_transducer_length_maxima": [_vp, _vp, _c_int, _vp, _vp],
+    "mi_transducer_profile_enable": [_c_int],
+    "mi_transducer_profile_read": [_c_int, ctypes.POINTER(_c_float), ctypes.POINTER(_c_int)],
+    "mi_transducer_profile_disable": [],
+    "mi_transducer_copy_probe": [_vp, _vp, _c_size_t, _vp],
 }  # fmt: skip
 
 EXPORTED_SYMBOLS = tuple(_SIGNATURES)
@@ -111,3 +116,24 @@ def workspace_bytes(B, T, U, D=0):
         # rnnt.py:184-185
         raise RuntimeError("Invalid parameter passed when calculating working space memory")
     return int(out.value)
+
+
+PROFILE_KERNELS = {"denom_gather_kernel": 0, "lattice_kernel": 1, "cell_kernel": 2, "grad_stream_kernel": 3}
+
+
+def profile_enable(max_launches):
+    check_status(lib().mi_transducer_profile_enable(int(max_launches)), "profile_enable")
+
+
+def profile_read():
+    """{kernel: (total_ms, launches)} for the launches recorded since the last read."""
+    out = {}
+    for name, kid in PROFILE_KERNELS.items():
+        ms, n = _c_float(0.0), _c_int(0)
+        check_status(lib().mi_transducer_profile_read(kid, ctypes.byref(ms), ctypes.byref(n)), "profile_read")
+        out[name] = (float(ms.value), int(n.value))
+    return out
+
+
+def profile_disable():
+    check_status(lib().mi_transducer_profile_disable(), "profile_disable")

@@ -28,7 +28,20 @@
 #include <math.h>
 #include <stdint.h>
 
+#include <vector>
+
 #include "mi_transducer.h"
+
+// Tunables of the two bandwidth passes (compile-time; the defaults are the measured best).
+#ifndef MI_XCD_MAP
+#define MI_XCD_MAP 1  // 1: each XCD streams one contiguous eighth of the (b,t) rows
+#endif
+#ifndef MI_NT_K1
+#define MI_NT_K1 0    // non-temporal loads in the long-row denominator pass
+#endif
+#ifndef MI_NT_K4
+#define MI_NT_K4 0    // non-temporal loads in the long-row gradient pass
+#endif
 
 namespace {
 
@@ -94,13 +107,12 @@ __device__ __forceinline__ float wave_sum(float v) {
 }
 
 __device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
-
-// Workgroup ids are dealt round-robin to the 8 XCDs; give each XCD one contiguous
-// eighth of the rows so that rows sharing a cache line meet in the same L2.
-__device__ __forceinline__ long long remap_block(long long chunk) {
-  const unsigned bid = blockIdx.x;
-  return (long long)(bid & 7u) * chunk + (long long)(bid >> 3);
-}
+#ifdef MI_EXPERIMENT_NO_EXP
+__device__ __forceinline__ float stream_exp2(float x) { return x * 1e-3f; }
+#else
+__device__ __forceinline__ float stream_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
+#endif
+__device__ __forceinline__ float clamp_sym(float g, float bound) { return fminf(fmaxf(g, -bound), bound); }
 
 // Element access for the three logit dtypes.  A "vector" is 16 bytes.
 template <int DT> struct Elem;
@@ -182,81 +194,193 @@ template <int DT> struct RowWindow {
   const uint4* vp;
   int mis;
   __device__ __forceinline__ RowWindow(const void* base, size_t first_elem) {
-    const uintptr_t a0 = (uintptr_t)base + first_elem * Elem<DT>::BYTES;
-    const uintptr_t al = a0 & ~(uintptr_t)15;
-    vp = (const uint4*)al;
-    mis = (int)((a0 - al) / Elem<DT>::BYTES);
+    const char* p = (const char*)base + first_elem * Elem<DT>::BYTES;
+    const int misbytes = (int)((uintptr_t)p & 15);
+    vp = (const uint4*)(p - misbytes);
+    mis = misbytes / Elem<DT>::BYTES;
+  }
+};
+
+// ----------------------------------------------------------------------------------------
+// Row streaming helpers shared by the two bandwidth passes.
+//
+// A row of VD elements starting at an arbitrary element offset is split into
+//   head : the elements before the first 16-byte boundary inside the row   (< VEC of them)
+//   body : nb whole aligned vectors, vector jb0 + i of the row's window     (the bulk)
+//   tail : what is left of the token logits after the last whole vector     (< VEC)
+// The body is moved with aligned 16-byte accesses, R vectors per lane in flight; head and
+// tail (and the D duration entries of a TDT row) are moved one element per lane.
+// ----------------------------------------------------------------------------------------
+typedef unsigned u32x4 __attribute__((ext_vector_type(4)));
+
+// streaming load: the logits are read exactly once per pass, keep them out of the caches' way
+template <bool NT> __device__ __forceinline__ uint4 load_stream(const uint4* p) {
+  if constexpr (NT) {
+    const u32x4 v = __builtin_nontemporal_load((const u32x4*)p);
+    return make_uint4(v.x, v.y, v.z, v.w);
+  } else {
+    return *p;
+  }
+}
+
+// Workgroups are dealt round-robin to the 8 XCDs in launch order.  The logical block id is
+// permuted so that each XCD takes MI_XCD_SPAN consecutive logical blocks (a contiguous piece
+// of the tensor) per turn: contiguous enough for the XCD's own L2 and TLB to see a linear
+// walk, fine enough that utterances of different lengths spread evenly over the XCDs.
+// MI_XCD_SPAN = 1 is the plain launch order.  The grid is a multiple of 8 * MI_XCD_SPAN.
+#ifndef MI_K1_REVERSE
+#define MI_K1_REVERSE 1
+#endif
+#ifndef MI_K4_REVERSE
+#define MI_K4_REVERSE 0
+#endif
+#ifndef MI_XCD_SPAN
+#define MI_XCD_SPAN 1024
+#endif
+__device__ __forceinline__ unsigned logical_block() {
+  const unsigned xcd = blockIdx.x & 7u, turn = blockIdx.x >> 3;
+  return (turn / MI_XCD_SPAN) * (8u * MI_XCD_SPAN) + xcd * MI_XCD_SPAN + (turn % MI_XCD_SPAN);
+}
+
+// Which (b, t, u) row a wave works on.  Grid = (8 * ceil(U/4), ceil(B*T/8)): workgroups are
+// dealt round-robin to the 8 XCDs in linear-id order, so blockIdx.x & 7 names the XCD; each
+// XCD gets a contiguous eighth of the (b,t) rows and walks it in memory order.  Rows are not
+// cache-line aligned, so neighbours share lines: keeping them in one L2 lets a gradient line
+// be completed before it is written back.
+struct RowId {
+  int b, t, u;
+  bool in_range;
+};
+__device__ __forceinline__ RowId row_of_wave(int T, int U, int BT, int bt_chunk) {
+  RowId id;
+#if MI_XCD_MAP
+  const unsigned xcd = blockIdx.x & 7u, ub = blockIdx.x >> 3;
+  const unsigned bt = xcd * (unsigned)bt_chunk + blockIdx.y;
+#else
+  const unsigned ub = blockIdx.x, bt = blockIdx.y;
+  (void)bt_chunk;
+#endif
+  id.u = __builtin_amdgcn_readfirstlane((int)(ub * kRowsPerBlock + (threadIdx.x >> 6)));
+  id.b = (int)(bt / (unsigned)T);
+  id.t = (int)(bt - (unsigned)id.b * (unsigned)T);
+  id.in_range = bt < (unsigned)BT && id.u < U;
+#if MI_XCD_MAP
+  id.in_range = id.in_range && blockIdx.y < (unsigned)bt_chunk;
+#endif
+  return id;
+}
+
+template <int DT> struct RowSplit {
+  int hc;   // head elements: row elements [0, hc)
+  int jb0;  // first whole vector of the window
+  int nb;   // whole vectors: row elements [hc, hc + nb*VEC)
+  int tc;   // tail elements: row elements [hc + nb*VEC, V)
+  __device__ __forceinline__ RowSplit(int mis, int V) {
+    constexpr int VEC = Elem<DT>::VEC;
+    hc = mis ? VEC - mis : 0;
+    if (hc > V) hc = V;
+    jb0 = mis ? 1 : 0;
+    nb = (V - hc) / VEC;
+    tc = V - hc - nb * VEC;
+  }
+  __device__ __forceinline__ int tail0() const { return hc + nb * Elem<DT>::VEC; }
+  // window index of whole vector j, clamped into the row so that any lane may load it
+  __device__ __forceinline__ int body_vector(int j) const { return nb > 0 ? jb0 + (j < nb ? j : nb - 1) : 0; }
+  // head and tail token elements are handled one per lane: lanes [0,hc) take the head, lanes
+  // [VEC, VEC+tc) the tail; -1 for every other lane
+  __device__ __forceinline__ int extra_token(int lane) const {
+    constexpr int VEC = Elem<DT>::VEC;
+    if (lane < hc) return lane;
+    if (lane >= VEC && lane < VEC + tc) return tail0() + lane - VEC;
+    return -1;
+  }
+};
+
+// running (max, sum of exp) of one lane, base-2 scaled: sum_i 2^(x_i*log2e - m*log2e)
+struct LaneLse {
+  float m, s;
+  __device__ __forceinline__ LaneLse() : m(-1.0e30f), s(0.f) {}
+  template <int N> __device__ __forceinline__ void add(const float* x) {
+    float cm = x[0];
+#pragma unroll
+    for (int i = 1; i < N; ++i) cm = fmaxf(cm, x[i]);
+    const float mnew = fmaxf(m, cm);  // never below -1e30: no inf - inf, and -mnew*log2e stays finite
+    const float off = -mnew * kLog2e;
+    float acc = 0.f;
+#pragma unroll
+    for (int i = 0; i < N; ++i) acc += fast_exp2(fmaf(x[i], kLog2e, off));
+    s = fmaf(s, fast_exp2((m - mnew) * kLog2e), acc);
+    m = mnew;
   }
 };
 
 // ----------------------------------------------------------------------------------------
 // Pass 1: denominators + gather (replaces reduce.py:121-248 and the per-step gathers of
-// logp() in gpu_rnnt_kernel.py:42-64).  One wave per (b,t,u) row; padded rows exit.
+// logp() in gpu_rnnt_kernel.py:42-64).  Grid (ceil(U/4), T, B), one wave per (b,t,u) row;
+// waves of padded rows exit at once.
 // ----------------------------------------------------------------------------------------
 template <int DT>
 __global__ __launch_bounds__(256) void denom_gather_kernel(
     const void* __restrict__ acts, const int64_t* __restrict__ labels, const int64_t* __restrict__ act_lens,
     const int64_t* __restrict__ label_lens, float* __restrict__ denom, float* __restrict__ arcs, int T, int U, int V,
-    int D, int blank, int ND, int Us, int A, long long rows, long long chunk) {
+    int D, int blank, int ND, int Us, int A, int BT, int bt_chunk) {
   constexpr int VEC = Elem<DT>::VEC;
   constexpr int R = 4;  // vectors in flight per lane
+  constexpr bool NT = MI_NT_K1 != 0;
   const int lane = threadIdx.x & 63;
-  const long long r =
-      __builtin_amdgcn_readfirstlane((int)(remap_block(chunk) * kRowsPerBlock + (threadIdx.x >> 6)));
-  if (r >= rows) return;
-  const int u = (int)(r % U);
-  const long long bt = r / U;
-  const int t = (int)(bt % T);
-  const int b = (int)(bt / T);
+  const RowId id = row_of_wave(T, U, BT, bt_chunk);
+  if (!id.in_range) return;
+  const int b = id.b, t = id.t, u = id.u;
   const int Tb = clampi(act_lens[b], 1, T);
   const int Ub = clampi(label_lens[b] + 1, 1, U);
   if (t >= Tb || u >= Ub) return;
 
   const int VD = V + D;
-  const RowWindow<DT> w(acts, (size_t)r * VD);
-  const int nvec = (w.mis + V + VEC - 1) / VEC;  // only the token logits enter the denominator
+  const size_t r = ((size_t)b * T + t) * U + u;
+  const size_t e0 = r * VD;
+  // the two gathered logits do not depend on the reduction: ask for them first
+  const int lab = (u < Ub - 1) ? clampi(labels[(size_t)b * (U - 1) + u], 0, V - 1) : -1;
+  const float xb = Elem<DT>::load1(acts, e0 + blank);
+  const float xl = Elem<DT>::load1(acts, e0 + (lab >= 0 ? lab : blank));
+  const float xd = (lane < D) ? Elem<DT>::load1(acts, e0 + V + lane) : kNegInf;
 
-  float m = kNegInf, s = 0.f;
-  for (int j0 = lane; j0 < nvec; j0 += 64 * R) {
+  const RowWindow<DT> w(acts, e0);
+  const RowSplit<DT> sp(w.mis, V);
+  // head and tail: one element per lane (lanes [0,hc) and [VEC, VEC+tc))
+  float xe = kNegInf;
+  if (lane < sp.hc) xe = Elem<DT>::load1(acts, e0 + lane);
+  else if (lane >= VEC && lane < VEC + sp.tc) xe = Elem<DT>::load1(acts, e0 + sp.tail0() + lane - VEC);
+
+  LaneLse acc;
+  const uint4* vp = w.vp + sp.jb0 + lane;
+  int rounds = sp.nb >> 6;
+  for (; rounds >= R; rounds -= R, vp += 64 * R) {
     uint4 raw[R];
 #pragma unroll
-    for (int k = 0; k < R; ++k) {
-      const int j = j0 + 64 * k;
-      if (j < nvec) raw[k] = w.vp[j];
-    }
-    float x[R][VEC];
-    float cm = kNegInf;
+    for (int k = 0; k < R; ++k) raw[k] = load_stream<NT>(vp + 64 * k);
+    float x[R * VEC];
 #pragma unroll
-    for (int k = 0; k < R; ++k) {
-      const int j = j0 + 64 * k;
-      Elem<DT>::unpack(raw[k], x[k]);
-#pragma unroll
-      for (int i = 0; i < VEC; ++i) {
-        const int v = j * VEC + i - w.mis;
-        if (j >= nvec || v < 0 || v >= V) x[k][i] = kNegInf;
-        cm = fmaxf(cm, x[k][i]);
-      }
-    }
-    const float mnew = fmaxf(m, cm);
-    if (mnew > kNegInf) {
-      float acc = 0.f;
-      const float off = -mnew * kLog2e;
-#pragma unroll
-      for (int k = 0; k < R; ++k)
-#pragma unroll
-        for (int i = 0; i < VEC; ++i) acc += fast_exp2(fmaf(x[k][i], kLog2e, off));
-      s = s * fast_exp2((m - mnew) * kLog2e) + acc;
-      m = mnew;
-    }
+    for (int k = 0; k < R; ++k) Elem<DT>::unpack(raw[k], x + k * VEC);
+    acc.add<R * VEC>(x);
   }
-  const float M = wave_max(m);
-  const float part = (m > kNegInf) ? s * fast_exp2((m - M) * kLog2e) : 0.f;
-  const float S = wave_sum(part);
+  for (; rounds > 0; --rounds, vp += 64) {
+    float x[VEC];
+    Elem<DT>::unpack(load_stream<NT>(vp), x);
+    acc.add<VEC>(x);
+  }
+  if (sp.nb & 63) {  // last, partial round of whole vectors
+    float x[VEC];
+#pragma unroll
+    for (int i = 0; i < VEC; ++i) x[i] = kNegInf;
+    if (lane < (sp.nb & 63)) Elem<DT>::unpack(load_stream<NT>(vp), x);
+    acc.add<VEC>(x);
+  }
+  acc.add<1>(&xe);
+
+  const float M = wave_max(acc.m);
+  const float S = wave_sum(acc.s * fast_exp2((acc.m - M) * kLog2e));
   const float dn = -M - logf(S);
 
-  const int lab = (u < Ub - 1) ? clampi(labels[(size_t)b * (U - 1) + u], 0, V - 1) : -1;
-  const float xb = Elem<DT>::load1(acts, (size_t)r * VD + blank);
-  const float xl = lab >= 0 ? Elem<DT>::load1(acts, (size_t)r * VD + lab) : 0.f;
   const size_t base = ((size_t)(b * ND + t + u) * A) * Us + u;
   if (lane == 0) {
     denom[r] = dn;
@@ -264,7 +388,6 @@ __global__ __launch_bounds__(256) void denom_gather_kernel(
     arcs[base + Us] = lab >= 0 ? xl + dn : 0.f;
   }
   if (D > 0) {  // duration log-softmax (rnnt_pytorch.py:568), one lane per duration
-    const float xd = lane < D ? Elem<DT>::load1(acts, (size_t)r * VD + V + lane) : kNegInf;
     const float dm = wave_max(xd);
     const float ds = wave_sum(lane < D ? expf(xd - dm) : 0.f);
     const float dden = -dm - logf(ds);
@@ -276,13 +399,27 @@ __global__ __launch_bounds__(256) void denom_gather_kernel(
 // Lattice helpers
 // ----------------------------------------------------------------------------------------
 // log(exp(a)+exp(b)) with the sum carried in fp64 and the correction term in fp32
-// (rnnt_helper.py:42-53: the other operand is returned when one is -inf).
+// (rnnt_helper.py:42-53: the other operand is returned when one is -inf).  Branch-free:
+// with one operand -inf the correction is log(1 + 2^-inf) = 0; only (-inf, -inf) needs the select.
 __device__ __forceinline__ double lse_h(double a, double b) {
   const double m = fmax(a, b);
   const double n = fmin(a, b);
-  if (n == -INFINITY) return m;
   const float d = (float)(n - m);
-  return m + (double)__logf(1.0f + __expf(d));
+  const double r = m + (double)(__builtin_amdgcn_logf(1.0f + fast_exp2(d * kLog2e)) * 0.6931471805599453f);
+  return (n == -INFINITY) ? m : r;
+}
+
+// value of the lane below / above (wave shift by one lane through DPP, no LDS round trip);
+// lane 0 / lane 63 receives `fill`
+__device__ __forceinline__ double from_lane_below(double v, double fill) {
+  const int lo = __builtin_amdgcn_update_dpp(__double2loint(fill), __double2loint(v), 0x138, 0xf, 0xf, false);
+  const int hi = __builtin_amdgcn_update_dpp(__double2hiint(fill), __double2hiint(v), 0x138, 0xf, 0xf, false);
+  return __hiloint2double(hi, lo);
+}
+__device__ __forceinline__ double from_lane_above(double v, double fill) {
+  const int lo = __builtin_amdgcn_update_dpp(__double2loint(fill), __double2loint(v), 0x130, 0xf, 0xf, false);
+  const int hi = __builtin_amdgcn_update_dpp(__double2hiint(fill), __double2hiint(v), 0x130, 0xf, 0xf, false);
+  return __hiloint2double(hi, lo);
 }
 
 template <int K> struct FloatK;
@@ -311,13 +448,37 @@ template <int K> __device__ __forceinline__ void load_k(const float* p, float* o
 
 template <int K> struct Prefetch { static constexpr int P = K <= 2 ? 8 : (K == 4 ? 4 : (K == 8 ? 2 : 1)); };
 
+template <int K> __device__ __forceinline__ void store_k(double* p, const double* v) {
+  typedef double d2 __attribute__((ext_vector_type(2)));
+  if constexpr (K == 1) {
+    p[0] = v[0];
+  } else {
+#pragma unroll
+    for (int q = 0; q < K / 2; ++q) {
+      d2 x;
+      x[0] = v[2 * q];
+      x[1] = v[2 * q + 1];
+      *(d2*)(p + 2 * q) = x;
+    }
+  }
+}
+
+// Arc log-probs of cells outside the utterance's lattice were never written: whatever bits
+// are there must not turn a -inf lattice value into NaN, so they are forced finite.
+__device__ __forceinline__ float finite_arc(float x) { return fminf(fmaxf(x, -3.0e38f), 3.0e38f); }
+
 // RNNT lattice: one wave per (utterance, direction).  Lane l owns columns u = l*K .. l*K+K-1
 // and, at step n, the cells (n-u, u) of anti-diagonal n.
 //   alpha (gpu_rnnt_kernel.py:73-172): every cell pushes e = alpha + lp_label to its right
 //   neighbour and s = alpha + lp_blank to the cell below; the next diagonal is lse(e_in, s_in).
 //   beta  (gpu_rnnt_kernel.py:175-269): pulled from the diagonal above.
-// The arc log-probs of diagonals n .. n+P-1 are prefetched into registers while the previous
-// P diagonals are being computed; they do not depend on the recursion.
+// No boundary tests in the loop: everything starts at -inf, the only finite source is
+// alpha(0,0) = 0 (resp. the corner beta(Tb-1,Ub-1) = lp_blank), and values only flow right/down
+// (resp. left/up), so cells outside the lattice either stay -inf (where they could feed a
+// valid cell) or hold junk that no valid cell ever reads.  Every lane stores its K values of
+// every diagonal: the skewed rows are 64*K wide.
+// The arc log-probs of P diagonals are fetched into registers while the previous P
+// diagonals are being computed; they do not depend on the recursion.
 template <int K>
 __global__ __launch_bounds__(64) void rnnt_lattice_kernel(const float* __restrict__ arcs, double* __restrict__ alphas,
                                                           double* __restrict__ betas, double* __restrict__ ll,
@@ -334,19 +495,20 @@ __global__ __launch_bounds__(64) void rnnt_lattice_kernel(const float* __restric
   const int Tb = clampi(act_lens[b], 1, T);
   const int Ub = clampi(label_lens[b] + 1, 1, U);
   const int nd = Tb + Ub - 1;
-  const float* arcs_b = arcs + (size_t)b * ND * A * Us + u0;
+  const size_t row_pitch = (size_t)A * Us;
+  const float* arcs_b = arcs + (size_t)b * ND * row_pitch + u0;
   const double NINF = -INFINITY;
 
-  float blk[P][K], lab[P][K];
+  // rows [n, n + step*P) of the blank and label planes, this lane's K columns (rows clamped into
+  // the utterance so that the loads never depend on a branch)
   auto load_rows = [&](int nfirst, int step, float(&Bk)[P][K], float(&Lb)[P][K]) {
 #pragma unroll
     for (int p = 0; p < P; ++p) {
-      const int n = nfirst + step * p;
-      if (n >= 0 && n < nd) {
-        const float* rp = arcs_b + (size_t)n * A * Us;
-        load_k<K>(rp, Bk[p]);
-        load_k<K>(rp + Us, Lb[p]);
-      }
+      int n = nfirst + step * p;
+      n = n < 0 ? 0 : (n >= nd ? nd - 1 : n);
+      const float* rp = arcs_b + (size_t)n * row_pitch;
+      load_k<K>(rp, Bk[p]);
+      load_k<K>(rp + Us, Lb[p]);
     }
   };
 
@@ -355,94 +517,90 @@ __global__ __launch_bounds__(64) void rnnt_lattice_kernel(const float* __restric
     double e[K], s[K];
 #pragma unroll
     for (int k = 0; k < K; ++k) e[k] = s[k] = NINF;
-    load_rows(0, 1, blk, lab);
-    for (int n0 = 0; n0 < nd; n0 += P) {
-      float nb[P][K], nl[P][K];
-      load_rows(n0 + P, 1, nb, nl);
+    if (lane == 0) s[0] = 0.0;  // makes alpha(0,0) = lse(-inf, 0) = 0
+    auto step_fn = [&](int n, const float* bk, const float* lb) {
+      const double left = from_lane_below(e[K - 1], NINF);
+      double a[K];
 #pragma unroll
-      for (int p = 0; p < P; ++p) {
-        const int n = n0 + p;
-        if (n < nd) {
-          double left = __shfl_up(e[K - 1], 1, 64);
-          if (lane == 0) left = NINF;
-          double a[K];
+      for (int k = 0; k < K; ++k) a[k] = lse_h(k == 0 ? left : e[k - 1], s[k]);
+      store_k<K>(out + (size_t)n * Us, a);
 #pragma unroll
-          for (int k = 0; k < K; ++k) {
-            const int u = u0 + k, t = n - u;
-            const bool valid = (u < Ub) && (t >= 0) && (t < Tb);
-            double v = lse_h(k == 0 ? left : e[k - 1], s[k]);
-            if (n == 0 && u == 0) v = 0.0;
-            a[k] = valid ? v : NINF;
-          }
-#pragma unroll
-          for (int k = 0; k < K; ++k) {
-            const int u = u0 + k, t = n - u;
-            const bool valid = (u < Ub) && (t >= 0) && (t < Tb);
-            e[k] = valid ? a[k] + (double)lab[p][k] : NINF;
-            s[k] = valid ? a[k] + (double)blk[p][k] : NINF;
-            if (valid) out[(size_t)n * Us + k] = a[k];
-            if (n == nd - 1 && u == Ub - 1 && valid) {  // llForward and the cost (rnnt_helper.py:106-116)
-              ll[2 * b] = s[k];
-              costs[b] = -(float)s[k] * cost_scale;
-            }
-          }
-        }
+      for (int k = 0; k < K; ++k) {
+        e[k] = a[k] + (double)finite_arc(lb[k]);
+        s[k] = a[k] + (double)finite_arc(bk[k]);
       }
+    };
+    float bufa_b[P][K], bufa_l[P][K], bufb_b[P][K], bufb_l[P][K];
+    int n0 = 0;
+    load_rows(0, 1, bufa_b, bufa_l);
+    for (; n0 + 2 * P <= nd; n0 += 2 * P) {
+      load_rows(n0 + P, 1, bufb_b, bufb_l);
+      __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-      for (int p = 0; p < P; ++p)
+      for (int p = 0; p < P; ++p) step_fn(n0 + p, bufa_b[p], bufa_l[p]);
+      load_rows(n0 + 2 * P, 1, bufa_b, bufa_l);
+      __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-        for (int k = 0; k < K; ++k) {
-          blk[p][k] = nb[p][k];
-          lab[p][k] = nl[p][k];
-        }
+      for (int p = 0; p < P; ++p) step_fn(n0 + P + p, bufb_b[p], bufb_l[p]);
     }
+    for (; n0 < nd; ++n0) {  // fewer than 2P diagonals left
+      float bk[K], lb[K];
+      const float* rp = arcs_b + (size_t)n0 * row_pitch;
+      load_k<K>(rp, bk);
+      load_k<K>(rp + Us, lb);
+      step_fn(n0, bk, lb);
+    }
+    // after the last diagonal the owner of column Ub-1 holds s = alpha(Tb-1,Ub-1) + lp_blank = llForward
+#pragma unroll
+    for (int k = 0; k < K; ++k)
+      if (u0 + k == Ub - 1) {
+        ll[2 * b] = s[k];
+        costs[b] = -(float)s[k] * cost_scale;  // rnnt_helper.py:106-116
+      }
   } else {
     double* out = betas + (size_t)b * ND * Us + u0;
     double bt[K];
+    // diagonal nd-1 holds the corner cell only: beta(Tb-1,Ub-1) = lp_blank(Tb-1,Ub-1)
+    {
+      float bk[K];
+      load_k<K>(arcs_b + (size_t)(nd - 1) * row_pitch, bk);
 #pragma unroll
-    for (int k = 0; k < K; ++k) bt[k] = NINF;
-    load_rows(nd - 1, -1, blk, lab);
-    for (int n0 = nd - 1; n0 >= 0; n0 -= P) {
-      float nb[P][K], nl[P][K];
-      load_rows(n0 - P, -1, nb, nl);
-#pragma unroll
-      for (int p = 0; p < P; ++p) {
-        const int n = n0 - p;
-        if (n >= 0) {
-          double right = __shfl_down(bt[0], 1, 64);
-          if (lane == 63) right = NINF;
-          double nv[K];
-#pragma unroll
-          for (int k = 0; k < K; ++k) {
-            const int u = u0 + k, t = n - u;
-            const bool valid = (u < Ub) && (t >= 0) && (t < Tb);
-            const double rgt = (k == K - 1) ? right : bt[k + 1];
-            const double em = (u + 1 < Ub) ? rgt + (double)lab[p][k] : NINF;
-            double ne;
-            if (t == Tb - 1)
-              ne = (u == Ub - 1) ? (double)blk[p][k] : NINF;
-            else
-              ne = bt[k] + (double)blk[p][k];
-            nv[k] = valid ? lse_h(em, ne) : NINF;
-          }
-#pragma unroll
-          for (int k = 0; k < K; ++k) {
-            const int u = u0 + k, t = n - u;
-            const bool valid = (u < Ub) && (t >= 0) && (t < Tb);
-            bt[k] = nv[k];
-            if (valid) out[(size_t)n * Us + k] = nv[k];
-            if (n == 0 && u == 0) ll[2 * b + 1] = nv[k];
-          }
-        }
-      }
-#pragma unroll
-      for (int p = 0; p < P; ++p)
-#pragma unroll
-        for (int k = 0; k < K; ++k) {
-          blk[p][k] = nb[p][k];
-          lab[p][k] = nl[p][k];
-        }
+      for (int k = 0; k < K; ++k) bt[k] = (u0 + k == Ub - 1) ? (double)bk[k] : NINF;
+      store_k<K>(out + (size_t)(nd - 1) * Us, bt);
     }
+    auto step_fn = [&](int n, const float* bk, const float* lb) {
+      const double right = from_lane_above(bt[0], NINF);
+      double nv[K];
+#pragma unroll
+      for (int k = 0; k < K; ++k) {
+        const double rgt = (k == K - 1) ? right : bt[k + 1];
+        nv[k] = lse_h(rgt + (double)finite_arc(lb[k]), bt[k] + (double)finite_arc(bk[k]));
+      }
+      store_k<K>(out + (size_t)n * Us, nv);
+#pragma unroll
+      for (int k = 0; k < K; ++k) bt[k] = nv[k];
+    };
+    float bufa_b[P][K], bufa_l[P][K], bufb_b[P][K], bufb_l[P][K];
+    int n0 = nd - 2;
+    load_rows(n0, -1, bufa_b, bufa_l);
+    for (; n0 - 2 * P + 1 >= 0; n0 -= 2 * P) {
+      load_rows(n0 - P, -1, bufb_b, bufb_l);
+      __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+      for (int p = 0; p < P; ++p) step_fn(n0 - p, bufa_b[p], bufa_l[p]);
+      load_rows(n0 - 2 * P, -1, bufa_b, bufa_l);
+      __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+      for (int p = 0; p < P; ++p) step_fn(n0 - P - p, bufb_b[p], bufb_l[p]);
+    }
+    for (; n0 >= 0; --n0) {
+      float bk[K], lb[K];
+      const float* rp = arcs_b + (size_t)n0 * row_pitch;
+      load_k<K>(rp, bk);
+      load_k<K>(rp + Us, lb);
+      step_fn(n0, bk, lb);
+    }
+    if (lane == 0) ll[2 * b + 1] = bt[0];  // beta(0,0)
   }
 }
 
@@ -586,8 +744,6 @@ __global__ __launch_bounds__(64) void tdt_lattice_kernel(const float* __restrict
 //                label id (-1 none, -2 padded cell), -, -, dlogit_0 .. dlogit_{D-1} }
 // where G_blank / G_label are the finished gradient entries of the two special logits.
 // ----------------------------------------------------------------------------------------
-__device__ __forceinline__ float clamp_sym(float g, float bound) { return fminf(fmaxf(g, -bound), bound); }
-
 __device__ __forceinline__ void write_coef(float* c, float dn, float W, float PB, float PL, float lpb, float lpl,
                                            int lab, int blank, float clamp, float scale) {
   float gb = expf(lpb) * W - PB;
@@ -698,96 +854,406 @@ __global__ __launch_bounds__(256) void tdt_cell_kernel(
 }
 
 // ----------------------------------------------------------------------------------------
-// Pass 2: the gradient stream.  One wave per row; reads V logits (valid rows only), writes
-// V + D gradient elements (every row).  Same kernel for RNNT (D = 0) and TDT.
-// zero_durations: the omega branch of TDT -- duration gradients are zero.
+// Pass 2: the gradient stream.  Grid (ceil(U/4), T, B), one wave per row; reads the V token
+// logits of valid rows, writes V + D gradient elements of every row.  Same kernel for RNNT
+// (D = 0) and TDT.  zero_durations: the omega branch of TDT -- duration gradients are zero.
 // ----------------------------------------------------------------------------------------
 template <int DT>
 __global__ __launch_bounds__(256) void grad_stream_kernel(const void* __restrict__ acts, void* __restrict__ grads,
-                                                          const float* __restrict__ coef, int V, int D, int blank,
-                                                          int CS, int zero_durations, long long rows,
-                                                          long long chunk) {
+                                                          const float* __restrict__ coef,
+                                                          const int64_t* __restrict__ act_lens,
+                                                          const int64_t* __restrict__ label_lens, int T, int U, int V,
+                                                          int D, int blank, int CS, int zero_durations, int BT,
+                                                          int bt_chunk) {
   constexpr int VEC = Elem<DT>::VEC;
   constexpr int R = 4;
+  constexpr bool NT = MI_NT_K4 != 0;
   const int lane = threadIdx.x & 63;
-  const long long r =
-      __builtin_amdgcn_readfirstlane((int)(remap_block(chunk) * kRowsPerBlock + (threadIdx.x >> 6)));
-  if (r >= rows) return;
+  const RowId id = row_of_wave(T, U, BT, bt_chunk);
+  if (!id.in_range) return;
+  const int b = id.b, t = id.t, u = id.u;
+  const int Tb = clampi(act_lens[b], 1, T);
+  const int Ub = clampi(label_lens[b] + 1, 1, U);
   const int VD = V + D;
-  const float* c = coef + (size_t)r * CS;
-  const int lab = __float_as_int(c[5]);
-  const RowWindow<DT> win(acts, (size_t)r * VD);
-  // acts and grads have the same shape and dtype; their bases may differ in alignment
-  const uintptr_t g0 = (uintptr_t)grads + (size_t)r * VD * Elem<DT>::BYTES;
-  const bool same_phase = ((g0 & 15) / Elem<DT>::BYTES) == (uintptr_t)win.mis;
-  uint4* gvp = (uint4*)(g0 & ~(uintptr_t)15);
-  const int mis = win.mis;
-  const int nvec = (mis + VD + VEC - 1) / VEC;
+  const size_t r = ((size_t)b * T + t) * U + u;
+  const size_t e0 = r * VD;
 
-  if (lab == -2) {  // padded cell: zeros
+  const RowWindow<DT> win(acts, e0);
+  const uintptr_t g0 = (uintptr_t)grads + e0 * Elem<DT>::BYTES;
+  uint4* gvp = (uint4*)(g0 & ~(uintptr_t)15);
+  // acts and grads have the same shape and dtype; their bases may still differ in alignment
+  const bool same_phase = (int)((g0 & 15) / Elem<DT>::BYTES) == win.mis;
+
+  if (t >= Tb || u >= Ub) {  // padded cell: zeros over all V + D entries
+    const RowSplit<DT> sp(win.mis, VD);
     const uint4 z = make_uint4(0, 0, 0, 0);
-    for (int j = lane; j < nvec; j += 64) {
-      const int first = j * VEC - mis;
-      if (same_phase && first >= 0 && first + VEC <= VD) {
-        gvp[j] = z;
-      } else {
-#pragma unroll
-        for (int i = 0; i < VEC; ++i) {
-          const int v = first + i;
-          if (v >= 0 && v < VD) Elem<DT>::store1(grads, (size_t)r * VD + v, 0.f);
-        }
-      }
+    if (same_phase) {
+      for (int i = lane; i < sp.nb; i += 64) gvp[sp.jb0 + i] = z;
+      if (lane < sp.hc) Elem<DT>::store1(grads, e0 + lane, 0.f);
+      else if (lane >= VEC && lane < VEC + sp.tc) Elem<DT>::store1(grads, e0 + sp.tail0() + lane - VEC, 0.f);
+    } else {
+      for (int v = lane; v < VD; v += 64) Elem<DT>::store1(grads, e0 + v, 0.f);
     }
     return;
   }
 
-  const float dl2 = c[0], W = c[1], cb = c[2], gB = c[3], gL = c[4];
+  const float* c = coef + r * CS;
+  const float4 c0 = *(const float4*)c;          // denom*log2e, W*scale, clamp bound, G_blank
+  const float2 c1 = *(const float2*)(c + 4);    // G_label, label id
+  const float dl2 = c0.x, W = c0.y, cb = c0.z, gB = c0.w, gL = c1.x;
+  const int lab = __float_as_int(c1.y);
   const bool clamp_on = cb < INFINITY;
-  for (int j0 = lane; j0 < nvec; j0 += 64 * R) {
+  const RowSplit<DT> sp(win.mis, V);
+
+  auto token_grad = [&](float x, int v) {
+    float g = fast_exp2(fmaf(x, kLog2e, dl2)) * W;
+    if (clamp_on) g = clamp_sym(g, cb);
+    if (v == blank) g = gB;
+    if (v == lab) g = gL;
+    return g;
+  };
+
+  // head, tail and duration entries: one element per lane
+  {
+    int v = -1;
+    if (lane < sp.hc) v = lane;
+    else if (lane >= VEC && lane < VEC + sp.tc) v = sp.tail0() + lane - VEC;
+    else if (lane >= 2 * VEC && lane < 2 * VEC + D) v = V + lane - 2 * VEC;
+    if (v >= 0) {
+      float g;
+      if (v < V) g = token_grad(Elem<DT>::load1(acts, e0 + v), v);
+      else g = zero_durations ? 0.f : c[kCoefBase + v - V];
+      Elem<DT>::store1(grads, e0 + v, g);
+    }
+  }
+
+  if (!same_phase) {  // never the case for two fresh torch tensors; correct but slow
+    for (int v = sp.hc + lane; v < sp.tail0(); v += 64)
+      Elem<DT>::store1(grads, e0 + v, token_grad(Elem<DT>::load1(acts, e0 + v), v));
+    return;
+  }
+
+  // whole vectors; the two special logits are patched in the one vector that holds them
+  const int jblank = (blank + win.mis) / VEC, jlab = lab >= 0 ? (lab + win.mis) / VEC : -1;
+  auto do_vector = [&](const uint4& raw, int j) {
+    float x[VEC], g[VEC];
+    Elem<DT>::unpack(raw, x);
+#pragma unroll
+    for (int i = 0; i < VEC; ++i) {
+      float gi = fast_exp2(fmaf(x[i], kLog2e, dl2)) * W;
+      if (clamp_on) gi = clamp_sym(gi, cb);
+      g[i] = gi;
+    }
+    if (j == jblank || j == jlab) {
+      const int first = j * VEC - win.mis;
+#pragma unroll
+      for (int i = 0; i < VEC; ++i) {
+        if (first + i == blank) g[i] = gB;
+        if (first + i == lab) g[i] = gL;
+      }
+    }
+    gvp[j] = Elem<DT>::pack(g);
+  };
+
+  int j = sp.jb0 + lane;
+  int rounds = sp.nb >> 6;
+  for (; rounds >= R; rounds -= R, j += 64 * R) {
     uint4 raw[R];
 #pragma unroll
-    for (int k = 0; k < R; ++k) {
-      const int j = j0 + 64 * k;
-      if (j < nvec) raw[k] = win.vp[j];
-    }
+    for (int k = 0; k < R; ++k) raw[k] = load_stream<NT>(win.vp + j + 64 * k);
+#pragma unroll
+    for (int k = 0; k < R; ++k) do_vector(raw[k], j + 64 * k);
+  }
+  for (; rounds > 0; --rounds, j += 64) do_vector(load_stream<NT>(win.vp + j), j);
+  if (lane < (sp.nb & 63)) do_vector(load_stream<NT>(win.vp + j), j);
+}
+
+// ----------------------------------------------------------------------------------------
+// Wave reductions through DPP (no LDS round trips): two quad permutes and two mirrors leave
+// every 16-lane row holding its own result in all lanes; the four row results are then read
+// into scalar registers and combined, so the value returned is wave-uniform.
+// ----------------------------------------------------------------------------------------
+template <int CTRL> __device__ __forceinline__ float dpp_f(float v) {
+  return __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), CTRL, 0xf, 0xf, true));
+}
+__device__ __forceinline__ float lane_value(float v, int lane) {
+  return __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), lane));
+}
+__device__ __forceinline__ float wave_max_u(float v) {
+  v = fmaxf(v, dpp_f<0xB1>(v));   // quad_perm [1,0,3,2]
+  v = fmaxf(v, dpp_f<0x4E>(v));   // quad_perm [2,3,0,1]
+  v = fmaxf(v, dpp_f<0x141>(v));  // row_half_mirror
+  v = fmaxf(v, dpp_f<0x140>(v));  // row_mirror
+  return fmaxf(fmaxf(lane_value(v, 0), lane_value(v, 16)), fmaxf(lane_value(v, 32), lane_value(v, 48)));
+}
+__device__ __forceinline__ float wave_sum_u(float v) {
+  v += dpp_f<0xB1>(v);
+  v += dpp_f<0x4E>(v);
+  v += dpp_f<0x141>(v);
+  v += dpp_f<0x140>(v);
+  return (lane_value(v, 0) + lane_value(v, 16)) + (lane_value(v, 32) + lane_value(v, 48));
+}
+
+// ----------------------------------------------------------------------------------------
+// The bandwidth passes for rows that fit in R vectors per lane (V <= 64*R*VEC, the usual
+// subword vocabularies).  A workgroup owns kChunkRows consecutive rows of one (b,t) -- one
+// contiguous piece of memory -- and each of its 4 waves walks rows wave, wave+4, ...; while a
+// row is being reduced the loads of the wave's next row are already in flight.
+// ----------------------------------------------------------------------------------------
+#ifndef MI_ROWS_PER_WAVE
+#define MI_ROWS_PER_WAVE 1
+#endif
+constexpr int kRowsPerWave = MI_ROWS_PER_WAVE;
+constexpr int kChunkRows = kRowsPerBlock * kRowsPerWave;
+
+// zero-fills elements [e_begin, e_end) of `base` with the whole workgroup: 16-byte stores on
+// the aligned middle, element stores on the ragged ends
+template <int DT> __device__ __forceinline__ void zero_elems(void* base, size_t e_begin, size_t e_end) {
+  constexpr int BYTES = Elem<DT>::BYTES;
+  if (e_begin >= e_end) return;
+  char* p0 = (char*)base + e_begin * BYTES;
+  char* p1 = (char*)base + e_end * BYTES;
+  const size_t len = (size_t)(p1 - p0);
+  size_t head = (16 - ((uintptr_t)p0 & 15)) & 15;
+  if (head > len) head = len;
+  const size_t tail = (len - head) & 15;
+  const size_t nvec = (len - head - tail) >> 4;
+  const int tid = threadIdx.x;
+  if (tid < (int)(head / BYTES)) Elem<DT>::store1(p0, tid, 0.f);
+  else if (tid >= 32 && tid - 32 < (int)(tail / BYTES)) Elem<DT>::store1(p1 - tail, tid - 32, 0.f);
+  uint4* q = (uint4*)(p0 + head);
+  const uint4 z = make_uint4(0, 0, 0, 0);
+  for (size_t i = tid; i < nvec; i += 256) q[i] = z;
+}
+
+template <int DT, int R>
+__global__ __launch_bounds__(256) void denom_rows_kernel(
+    const void* __restrict__ acts, const int64_t* __restrict__ labels, const int64_t* __restrict__ act_lens,
+    const int64_t* __restrict__ label_lens, float* __restrict__ denom, float* __restrict__ arcs, int T, int U, int V,
+    int D, int blank, int ND, int Us, int A, int nchunks, int nblocks) {
+  constexpr int VEC = Elem<DT>::VEC;
+  const int lane = threadIdx.x & 63;
+  const int wave = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
+  // 1-D grid over (b,t,chunk), chunk fastest = memory order
+  unsigned wg = logical_block();
+  if (wg >= (unsigned)nblocks) return;
+#if MI_K1_REVERSE
+  wg = (unsigned)nblocks - 1u - wg;
+#endif
+  const unsigned bt = wg / (unsigned)nchunks, chunk = wg - bt * (unsigned)nchunks;
+  const int b = (int)(bt / (unsigned)T), t = (int)(bt - (unsigned)b * (unsigned)T);
+  const int Tb = clampi(act_lens[b], 1, T);
+  const int Ub = clampi(label_lens[b] + 1, 1, U);
+  if (t >= Tb) return;
+  const int u_begin = (int)chunk * kChunkRows + wave;
+  const int u_end = min(Ub, (int)(chunk + 1) * kChunkRows);
+  if (u_begin >= u_end) return;
+  const int VD = V + D;
+  const size_t cell0 = ((size_t)b * T + t) * U;
+
+  // the wave's label ids, fetched once so that no row waits on an id before asking for its logit
+  int labs[kRowsPerWave];
+#pragma unroll
+  for (int i = 0; i < kRowsPerWave; ++i) {
+    const int uu = u_begin + kRowsPerBlock * i;
+    labs[i] = (uu < Ub - 1) ? clampi(labels[(size_t)b * (U - 1) + uu], 0, V - 1) : -1;
+  }
+
+  struct Row {
+    uint4 raw[R];
+    float xe, xb, xl, xd;
+    int mis;
+  };
+  auto fetch = [&](int uu, int lab, Row& d) {
+    const size_t e0 = (cell0 + uu) * VD;
+    const RowWindow<DT> w(acts, e0);
+    const RowSplit<DT> sp(w.mis, V);
+    d.mis = w.mis;
+    // every load is unconditional (out-of-range lanes re-read an in-row address and are masked
+    // later): loads under a branch would force the wait counters to drain at every join
+#pragma unroll
+    for (int k = 0; k < R; ++k) d.raw[k] = load_stream<MI_NT_K1 != 0>(w.vp + sp.body_vector(lane + 64 * k));
+    const int ve = sp.extra_token(lane);
+    d.xe = Elem<DT>::load1(acts, e0 + (ve >= 0 ? ve : blank));
+    d.xb = Elem<DT>::load1(acts, e0 + blank);
+    d.xl = Elem<DT>::load1(acts, e0 + (lab >= 0 ? lab : blank));
+    d.xd = Elem<DT>::load1(acts, e0 + (lane < D ? V + lane : blank));
+  };
+  auto reduce = [&](int uu, int lab, const Row& d) {
+    const RowSplit<DT> sp(d.mis, V);
+    const int full = sp.nb >> 6, rem = sp.nb & 63;
+    float x[R][VEC];
 #pragma unroll
     for (int k = 0; k < R; ++k) {
-      const int j = j0 + 64 * k;
-      if (j < nvec) {
+      Elem<DT>::unpack(d.raw[k], x[k]);
+      if (k >= full) {  // wave-uniform: the last, partly filled slot and the unused ones
+        const bool ok = (k == full) && (lane < rem);
+#pragma unroll
+        for (int i = 0; i < VEC; ++i) x[k][i] = ok ? x[k][i] : kNegInf;
+      }
+    }
+    const float xe = sp.extra_token(lane) >= 0 ? d.xe : kNegInf;
+    float cm = xe;
+#pragma unroll
+    for (int k = 0; k < R; ++k)
+#pragma unroll
+      for (int i = 0; i < VEC; ++i) cm = fmaxf(cm, x[k][i]);
+    const float M = wave_max_u(cm);
+    const float off = -M * kLog2e;
+    float acc = stream_exp2(fmaf(xe, kLog2e, off));
+#pragma unroll
+    for (int k = 0; k < R; ++k)
+#pragma unroll
+      for (int i = 0; i < VEC; ++i) acc += stream_exp2(fmaf(x[k][i], kLog2e, off));
+    const float S = wave_sum_u(acc);
+    const float dn = -M - __builtin_amdgcn_logf(S) * 0.6931471805599453f;
+
+    const size_t base = ((size_t)(b * ND + t + uu) * A) * Us + uu;
+    if (lane == 0) {
+      denom[cell0 + uu] = dn;
+      arcs[base] = d.xb + dn;
+      arcs[base + Us] = lab >= 0 ? d.xl + dn : 0.f;
+    }
+    if (D > 0) {  // duration log-softmax (rnnt_pytorch.py:568), one lane per duration
+      const float xd = lane < D ? d.xd : kNegInf;
+      const float dm = wave_max_u(xd);
+      const float ds = wave_sum_u(lane < D ? expf(xd - dm) : 0.f);
+      const float dden = -dm - logf(ds);
+      if (lane < D) arcs[base + (size_t)(2 + lane) * Us] = xd + dden;
+    }
+  };
+
+  Row cur, nxt;
+  fetch(u_begin, labs[0], cur);
+#pragma unroll
+  for (int i = 0; i < kRowsPerWave; ++i) {
+    const int uu = u_begin + kRowsPerBlock * i;
+    if (uu >= u_end) break;
+    if (i + 1 < kRowsPerWave) {
+      // always fetch (the last row of the wave re-reads itself): an unconditional load keeps the
+      // wait counters exact, so reducing row i never waits for the loads of row i+1
+      const bool more = uu + kRowsPerBlock < u_end;
+      fetch(more ? uu + kRowsPerBlock : uu, more ? labs[i + 1] : labs[i], nxt);
+    }
+    reduce(uu, labs[i], cur);
+    cur = nxt;
+  }
+}
+
+template <int DT, int R>
+__global__ __launch_bounds__(256) void grad_rows_kernel(const void* __restrict__ acts, void* __restrict__ grads,
+                                                        const float* __restrict__ coef,
+                                                        const int64_t* __restrict__ act_lens,
+                                                        const int64_t* __restrict__ label_lens, int T, int U, int V,
+                                                        int D, int blank, int CS, int zero_durations, int nchunks,
+                                                        int nblocks) {
+  constexpr int VEC = Elem<DT>::VEC;
+  const int lane = threadIdx.x & 63;
+  const int wave = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
+  // 1-D grid over (b,t,chunk), chunk fastest = memory order
+  unsigned wg = logical_block();
+  if (wg >= (unsigned)nblocks) return;
+#if MI_K4_REVERSE
+  wg = (unsigned)nblocks - 1u - wg;
+#endif
+  const unsigned bt = wg / (unsigned)nchunks, chunk = wg - bt * (unsigned)nchunks;
+  const int b = (int)(bt / (unsigned)T), t = (int)(bt - (unsigned)b * (unsigned)T);
+  const int Tb = clampi(act_lens[b], 1, T);
+  const int Ub = clampi(label_lens[b] + 1, 1, U);
+  const int VD = V + D;
+  const size_t cell0 = ((size_t)b * T + t) * U;
+  const int c0 = (int)chunk * kChunkRows;
+  const int c1 = min(U, c0 + kChunkRows);
+  // rows [c0, z0) of this chunk carry a gradient, rows [z0, c1) are padding: one contiguous range of zeros
+  const int z0 = (t >= Tb) ? c0 : max(c0, min(Ub, c1));
+  zero_elems<DT>(grads, (cell0 + z0) * VD, (cell0 + c1) * VD);
+  const int u_begin = c0 + wave;
+  if (u_begin >= z0) return;
+
+  struct Row {
+    uint4 raw[R];
+    float4 ca;
+    float2 cb;
+    float xe, gd;
+    int mis;
+  };
+  // head, tail and duration entries of a row: one element per lane
+  auto extra_index = [&](const RowSplit<DT>& sp) {
+    int v = -1;
+    if (lane < sp.hc) v = lane;
+    else if (lane >= VEC && lane < VEC + sp.tc) v = sp.tail0() + lane - VEC;
+    else if (lane >= 2 * VEC && lane < 2 * VEC + D) v = V + lane - 2 * VEC;
+    return v;
+  };
+  auto fetch = [&](int uu, Row& d) {
+    const size_t e0 = (cell0 + uu) * VD;
+    const RowWindow<DT> w(acts, e0);
+    const RowSplit<DT> sp(w.mis, V);
+    d.mis = w.mis;
+    // unconditional loads, as in the denominator pass
+#pragma unroll
+    for (int k = 0; k < R; ++k) d.raw[k] = load_stream<MI_NT_K4 != 0>(w.vp + sp.body_vector(lane + 64 * k));
+    const float* c = coef + (cell0 + uu) * CS;
+    d.ca = *(const float4*)c;        // denom*log2e, W*scale, clamp bound, G_blank
+    d.cb = *(const float2*)(c + 4);  // G_label, label id
+    const int v = extra_index(sp);
+    d.xe = Elem<DT>::load1(acts, e0 + ((v >= 0 && v < V) ? v : blank));
+    d.gd = c[v >= V ? kCoefBase + v - V : 0];
+  };
+  auto emit = [&](int uu, const Row& d) {
+    const size_t e0 = (cell0 + uu) * VD;
+    const RowSplit<DT> sp(d.mis, V);
+    const float dl2 = d.ca.x, W = d.ca.y, cb = d.ca.z, gB = d.ca.w, gL = d.cb.x;
+    const int lab = __float_as_int(d.cb.y);
+    const bool clamp_on = cb < INFINITY;
+    char* grow = (char*)grads + e0 * Elem<DT>::BYTES;  // same 16-byte phase as the acts row
+    uint4* gvp = (uint4*)(grow - d.mis * Elem<DT>::BYTES) + sp.jb0 + lane;
+    const int jblank = (blank + d.mis) / VEC - sp.jb0, jlab = lab >= 0 ? (lab + d.mis) / VEC - sp.jb0 : -1;
+#pragma unroll
+    for (int k = 0; k < R; ++k) {
+      const int j = lane + 64 * k;  // whole vector j of the row
+      if (j < sp.nb) {
         float x[VEC], g[VEC];
-        Elem<DT>::unpack(raw[k], x);
-        const int first = j * VEC - mis;
+        Elem<DT>::unpack(d.raw[k], x);
 #pragma unroll
         for (int i = 0; i < VEC; ++i) {
-          float gi = fast_exp2(fmaf(x[i], kLog2e, dl2)) * W;
+          float gi = stream_exp2(fmaf(x[i], kLog2e, dl2)) * W;
           if (clamp_on) gi = clamp_sym(gi, cb);
           g[i] = gi;
         }
-        if (blank >= first && blank < first + VEC) {
-#pragma unroll
-          for (int i = 0; i < VEC; ++i)
-            if (first + i == blank) g[i] = gB;
-        }
-        if (lab >= first && lab < first + VEC) {
-#pragma unroll
-          for (int i = 0; i < VEC; ++i)
-            if (first + i == lab) g[i] = gL;
-        }
-        if (same_phase && first >= 0 && first + VEC <= V) {
-          gvp[j] = Elem<DT>::pack(g);
-        } else {
+        if (j == jblank || j == jlab) {  // the two special logits are patched in the vector that holds them
+          const int first = sp.hc + j * VEC;
 #pragma unroll
           for (int i = 0; i < VEC; ++i) {
-            const int v = first + i;
-            if (v >= 0 && v < V) {
-              Elem<DT>::store1(grads, (size_t)r * VD + v, g[i]);
-            } else if (v >= V && v < VD) {
-              Elem<DT>::store1(grads, (size_t)r * VD + v, zero_durations ? 0.f : c[kCoefBase + v - V]);
-            }
+            if (first + i == blank) g[i] = gB;
+            if (first + i == lab) g[i] = gL;
           }
         }
+        gvp[64 * k] = Elem<DT>::pack(g);
       }
     }
+    const int v = extra_index(sp);
+    if (v >= 0) {
+      float g = zero_durations ? 0.f : d.gd;
+      if (v < V) {
+        g = stream_exp2(fmaf(d.xe, kLog2e, dl2)) * W;
+        if (clamp_on) g = clamp_sym(g, cb);
+        if (v == blank) g = gB;
+        if (v == lab) g = gL;
+      }
+      Elem<DT>::store1(grads, e0 + v, g);
+    }
+  };
+
+  Row cur, nxt;
+  fetch(u_begin, cur);
+#pragma unroll
+  for (int i = 0; i < kRowsPerWave; ++i) {
+    const int uu = u_begin + kRowsPerBlock * i;
+    if (uu >= z0) break;
+    if (i + 1 < kRowsPerWave) fetch(uu + kRowsPerBlock < z0 ? uu + kRowsPerBlock : uu, nxt);
+    emit(uu, cur);
+    cur = nxt;
   }
 }
 
@@ -853,6 +1319,43 @@ __global__ __launch_bounds__(256) void length_maxima_kernel(const int64_t* __res
 // ----------------------------------------------------------------------------------------
 // Host side
 // ----------------------------------------------------------------------------------------
+// Benchmark aid: while enabled, every launch of a pipeline kernel is bracketed by a pair of
+// HIP events on the stream it is launched on, so a harness can read per-kernel durations
+// of the very launches it timed.  Off by default; the events are created when it is enabled.
+struct ProfState {
+  bool on = false;
+  int cap = 0;
+  int count[MI_PROFILE_KERNELS] = {0, 0, 0, 0};
+  std::vector<hipEvent_t> start[MI_PROFILE_KERNELS], stop[MI_PROFILE_KERNELS];
+};
+ProfState g_prof;
+
+struct ProfScope {
+  int id;
+  hipStream_t stream;
+  bool live;
+  ProfScope(int kernel_id, hipStream_t s) : id(kernel_id), stream(s), live(false) {
+    if (g_prof.on && g_prof.count[id] < g_prof.cap) {
+      live = true;
+      (void)hipEventRecord(g_prof.start[id][g_prof.count[id]], stream);
+    }
+  }
+  ~ProfScope() {
+    if (live) {
+      (void)hipEventRecord(g_prof.stop[id][g_prof.count[id]], stream);
+      ++g_prof.count[id];
+    }
+  }
+};
+
+// Plain 16-byte copy, grid-stride: the yardstick for the HBM counters and for the copy
+// bandwidth this GPU actually reaches.
+__global__ __launch_bounds__(256) void copy_probe_kernel(const uint4* __restrict__ src, uint4* __restrict__ dst,
+                                                         size_t nvec) {
+  const size_t stride = (size_t)gridDim.x * blockDim.x;
+  for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < nvec; i += stride) dst[i] = src[i];
+}
+
 struct Common {
   const void* acts;
   int dt;
@@ -871,7 +1374,7 @@ int check_common(const void* acts, int dt, const int64_t* labels, const int64_t*
   if (V <= 0 || blank < 0 || blank >= V) return MI_TRANSDUCER_INVALID_VALUE;
   if (!make_layout(B, T, U, D, &c->L)) return MI_TRANSDUCER_INVALID_VALUE;
   if (ws_bytes < c->L.total || ((uintptr_t)ws & 255)) return MI_TRANSDUCER_INVALID_VALUE;
-  if ((long long)B * T * U > 0x7fffffffLL) return MI_TRANSDUCER_INVALID_VALUE;  // row index is kept in 31 bits
+  if ((long long)B * T > 65535LL * 8) return MI_TRANSDUCER_INVALID_VALUE;  // grid-size limit of the long-row kernels
   c->acts = acts; c->dt = dt; c->labels = labels; c->act_lens = act_lens; c->label_lens = label_lens;
   c->B = B; c->T = T; c->U = U; c->V = V; c->D = D; c->blank = blank;
   c->ws = (char*)ws; c->stream = (hipStream_t)stream;
@@ -896,26 +1399,73 @@ int make_tdt_params(int D, const int32_t* durations, float sigma, TdtParams* p) 
 
 inline int launch_status() { return hipGetLastError() == hipSuccess ? MI_TRANSDUCER_SUCCESS : MI_TRANSDUCER_LAUNCH_FAILURE; }
 
-void stream_grid(long long rows, unsigned* grid, long long* chunk) {
-  const long long nblk = (rows + kRowsPerBlock - 1) / kRowsPerBlock;
-  *chunk = (nblk + 7) / 8;
-  *grid = (unsigned)(*chunk * 8);
+struct RowGrid {
+  dim3 grid;
+  int BT, bt_chunk;
+};
+inline RowGrid row_grid(const Common& c) {
+  RowGrid g;
+  const unsigned ublocks = (unsigned)((c.U + kRowsPerBlock - 1) / kRowsPerBlock);
+  g.BT = c.B * c.T;
+#if MI_XCD_MAP
+  g.bt_chunk = (g.BT + 7) / 8;
+  g.grid = dim3(8 * ublocks, (unsigned)g.bt_chunk, 1);
+#else
+  g.bt_chunk = g.BT;
+  g.grid = dim3(ublocks, (unsigned)g.BT, 1);
+#endif
+  return g;
+}
+
+// smallest R in {1,2,4,8} with floor(V / VEC) <= 64*R, or 0 if the rows are too long for the
+// register-resident kernels
+#ifndef MI_USE_ROWS
+#define MI_USE_ROWS 1
+#endif
+inline int rows_R(const Common& c) {
+  if (!MI_USE_ROWS) return 0;
+  const int vec = c.dt == MI_DTYPE_F32 ? 4 : 8;
+  const int nb = c.V / vec;
+  for (int r = 1; r <= 8; r *= 2)
+    if (nb <= 64 * r) return r;
+  return 0;
+}
+inline int chunks_of(const Common& c) { return (c.U + kChunkRows - 1) / kChunkRows; }
+inline int chunk_blocks(const Common& c) { return chunks_of(c) * c.B * c.T; }
+// rounded up to whole turns of the XCD permutation
+inline dim3 chunk_grid(const Common& c) {
+  const unsigned turn = 8u * MI_XCD_SPAN;
+  return dim3(((unsigned)chunk_blocks(c) + turn - 1) / turn * turn, 1, 1);
 }
 
 int run_denom(const Common& c) {
   const Layout& L = c.L;
-  const long long rows = (long long)c.B * c.T * c.U;
-  unsigned grid; long long chunk;
-  stream_grid(rows, &grid, &chunk);
   float* denom = (float*)(c.ws + L.off_denom);
   float* arcs = (float*)(c.ws + L.off_arcs);
+  const RowGrid g = row_grid(c);
+  const int R = rows_R(c);
+  ProfScope prof(MI_PROFILE_DENOM, c.stream);
+#define LAUNCH_DENOM_ROWS(DT, RR)                                                                                   \
+  hipLaunchKernelGGL((denom_rows_kernel<DT, RR>), chunk_grid(c), dim3(256), 0, c.stream, c.acts, c.labels,           \
+                     c.act_lens, c.label_lens, denom, arcs, c.T, c.U, c.V, c.D, c.blank, L.ND, L.Us, L.A, chunks_of(c), chunk_blocks(c))
 #define LAUNCH_DENOM(DT)                                                                                            \
-  hipLaunchKernelGGL(denom_gather_kernel<DT>, dim3(grid), dim3(256), 0, c.stream, c.acts, c.labels, c.act_lens,      \
-                     c.label_lens, denom, arcs, c.T, c.U, c.V, c.D, c.blank, L.ND, L.Us, L.A, rows, chunk)
+  do {                                                                                                              \
+    switch (R) {                                                                                                    \
+      case 1: LAUNCH_DENOM_ROWS(DT, 1); break;                                                                      \
+      case 2: LAUNCH_DENOM_ROWS(DT, 2); break;                                                                      \
+      case 4: LAUNCH_DENOM_ROWS(DT, 4); break;                                                                      \
+      case 8: LAUNCH_DENOM_ROWS(DT, 8); break;                                                                      \
+      default:                                                                                                      \
+        hipLaunchKernelGGL(denom_gather_kernel<DT>, g.grid, dim3(256), 0, c.stream, c.acts, c.labels, c.act_lens,   \
+                           c.label_lens, denom, arcs, c.T, c.U, c.V, c.D, c.blank, L.ND, L.Us, L.A, g.BT,           \
+                           g.bt_chunk);                                                                             \
+    }                                                                                                               \
+  } while (0)
   if (c.dt == MI_DTYPE_F32) LAUNCH_DENOM(MI_DTYPE_F32);
   else if (c.dt == MI_DTYPE_BF16) LAUNCH_DENOM(MI_DTYPE_BF16);
   else LAUNCH_DENOM(MI_DTYPE_F16);
 #undef LAUNCH_DENOM
+#undef LAUNCH_DENOM_ROWS
   return launch_status();
 }
 
@@ -929,6 +1479,7 @@ int run_rnnt_lattice(const Common& c, float* costs, float lambda, int with_betas
   double* betas = (double*)(c.ws + L.off_betas);
   double* ll = (double*)(c.ws + L.off_ll);
   const unsigned grid = (unsigned)(with_betas ? 2 * c.B : c.B);
+  ProfScope prof(MI_PROFILE_LATTICE, c.stream);
 #define LAUNCH_LAT(KK)                                                                                               \
   hipLaunchKernelGGL(rnnt_lattice_kernel<KK>, dim3(grid), dim3(64), 0, c.stream, arcs, alphas, betas, ll, costs,      \
                      c.act_lens, c.label_lens, c.T, c.U, L.ND, L.A, cost_scale_of(lambda), with_betas)
@@ -952,6 +1503,7 @@ int run_tdt_lattice(const Common& c, float* costs, float lambda, int with_betas,
   const unsigned grid = (unsigned)(with_betas ? 2 * c.B : c.B);
   const size_t lds = (size_t)2 * prm.R * L.Us * sizeof(double);
   if (lds > 160 * 1024) return MI_TRANSDUCER_INVALID_VALUE;
+  ProfScope prof(MI_PROFILE_LATTICE, c.stream);
 #define LAUNCH_TLAT(KK)                                                                                              \
   do {                                                                                                               \
     if (lds > 48 * 1024 &&                                                                                           \
@@ -974,17 +1526,32 @@ int run_tdt_lattice(const Common& c, float* costs, float lambda, int with_betas,
 
 int run_grad_stream(const Common& c, void* grads, int zero_durations) {
   const Layout& L = c.L;
-  const long long rows = (long long)c.B * c.T * c.U;
-  unsigned grid; long long chunk;
-  stream_grid(rows, &grid, &chunk);
   const float* coef = (const float*)(c.ws + L.off_coef);
-#define LAUNCH_GRAD(DT)                                                                                              \
-  hipLaunchKernelGGL(grad_stream_kernel<DT>, dim3(grid), dim3(256), 0, c.stream, c.acts, grads, coef, c.V, c.D,       \
-                     c.blank, L.CS, zero_durations, rows, chunk)
+  const RowGrid g = row_grid(c);
+  // the row kernels store gradient vectors at the 16-byte phase of the logits row
+  const bool same_phase = (((uintptr_t)c.acts ^ (uintptr_t)grads) & 15) == 0;
+  const int R = same_phase ? rows_R(c) : 0;
+  ProfScope prof(MI_PROFILE_GRAD, c.stream);
+#define LAUNCH_GRAD_ROWS(DT, RR)                                                                                    \
+  hipLaunchKernelGGL((grad_rows_kernel<DT, RR>), chunk_grid(c), dim3(256), 0, c.stream, c.acts, grads, coef,         \
+                     c.act_lens, c.label_lens, c.T, c.U, c.V, c.D, c.blank, L.CS, zero_durations, chunks_of(c), chunk_blocks(c))
+#define LAUNCH_GRAD(DT)                                                                                             \
+  do {                                                                                                              \
+    switch (R) {                                                                                                    \
+      case 1: LAUNCH_GRAD_ROWS(DT, 1); break;                                                                       \
+      case 2: LAUNCH_GRAD_ROWS(DT, 2); break;                                                                       \
+      case 4: LAUNCH_GRAD_ROWS(DT, 4); break;                                                                       \
+      case 8: LAUNCH_GRAD_ROWS(DT, 8); break;                                                                       \
+      default:                                                                                                      \
+        hipLaunchKernelGGL(grad_stream_kernel<DT>, g.grid, dim3(256), 0, c.stream, c.acts, grads, coef, c.act_lens, \
+                           c.label_lens, c.T, c.U, c.V, c.D, c.blank, L.CS, zero_durations, g.BT, g.bt_chunk);      \
+    }                                                                                                               \
+  } while (0)
   if (c.dt == MI_DTYPE_F32) LAUNCH_GRAD(MI_DTYPE_F32);
   else if (c.dt == MI_DTYPE_BF16) LAUNCH_GRAD(MI_DTYPE_BF16);
   else LAUNCH_GRAD(MI_DTYPE_F16);
 #undef LAUNCH_GRAD
+#undef LAUNCH_GRAD_ROWS
   return launch_status();
 }
 
@@ -992,6 +1559,7 @@ int run_rnnt_cells(const Common& c, const float* grad_scale, float lambda, float
   const Layout& L = c.L;
   const long long cells = (long long)c.B * c.T * c.U;
   const unsigned grid = (unsigned)((cells + 255) / 256);
+  ProfScope prof(MI_PROFILE_CELL, c.stream);
   hipLaunchKernelGGL(rnnt_cell_kernel, dim3(grid), dim3(256), 0, c.stream, (const float*)(c.ws + L.off_denom),
                      (const float*)(c.ws + L.off_arcs), (const double*)(c.ws + L.off_alphas),
                      (const double*)(c.ws + L.off_betas), (const double*)(c.ws + L.off_ll), c.labels, c.act_lens,
@@ -1004,6 +1572,7 @@ int run_tdt_cells(const Common& c, const float* grad_scale, float lambda, float 
   const Layout& L = c.L;
   const long long cells = (long long)c.B * c.T * c.U;
   const unsigned grid = (unsigned)((cells + 255) / 256);
+  ProfScope prof(MI_PROFILE_CELL, c.stream);
   hipLaunchKernelGGL(tdt_cell_kernel, dim3(grid), dim3(256), 0, c.stream, (const float*)(c.ws + L.off_denom),
                      (const float*)(c.ws + L.off_arcs), (const double*)(c.ws + L.off_alphas),
                      (const double*)(c.ws + L.off_betas), (const double*)(c.ws + L.off_ll), c.labels, c.act_lens,
@@ -1134,6 +1703,56 @@ int mi_transducer_length_maxima(const int64_t* act_lens, const int64_t* label_le
                                 void* stream) {
   if (!act_lens || !label_lens || !out || B <= 0) return MI_TRANSDUCER_INVALID_VALUE;
   hipLaunchKernelGGL(length_maxima_kernel, dim3(1), dim3(256), 0, (hipStream_t)stream, act_lens, label_lens, B, out);
+  return launch_status();
+}
+
+int mi_transducer_profile_enable(int max_launches) {
+  if (max_launches <= 0 || max_launches > 65536) return MI_TRANSDUCER_INVALID_VALUE;
+  g_prof.on = false;
+  for (int k = 0; k < MI_PROFILE_KERNELS; ++k) {
+    while ((int)g_prof.start[k].size() < max_launches) {
+      hipEvent_t a, b;
+      if (hipEventCreate(&a) != hipSuccess || hipEventCreate(&b) != hipSuccess) return MI_TRANSDUCER_LAUNCH_FAILURE;
+      g_prof.start[k].push_back(a);
+      g_prof.stop[k].push_back(b);
+    }
+    g_prof.count[k] = 0;
+  }
+  g_prof.cap = max_launches;
+  g_prof.on = true;
+  return MI_TRANSDUCER_SUCCESS;
+}
+
+int mi_transducer_profile_read(int kernel_id, float* total_ms, int* launches) {
+  if (kernel_id < 0 || kernel_id >= MI_PROFILE_KERNELS || !total_ms || !launches) return MI_TRANSDUCER_INVALID_VALUE;
+  float total = 0.f;
+  const int n = g_prof.count[kernel_id];
+  for (int i = 0; i < n; ++i) {
+    float ms = 0.f;
+    if (hipEventSynchronize(g_prof.stop[kernel_id][i]) != hipSuccess ||
+        hipEventElapsedTime(&ms, g_prof.start[kernel_id][i], g_prof.stop[kernel_id][i]) != hipSuccess)
+      return MI_TRANSDUCER_LAUNCH_FAILURE;
+    total += ms;
+  }
+  *total_ms = total;
+  *launches = n;
+  g_prof.count[kernel_id] = 0;
+  return MI_TRANSDUCER_SUCCESS;
+}
+
+int mi_transducer_profile_disable(void) {
+  g_prof.on = false;
+  return MI_TRANSDUCER_SUCCESS;
+}
+
+int mi_transducer_copy_probe(const void* src, void* dst, size_t bytes, void* stream) {
+  if (!src || !dst || bytes == 0 || (bytes & 15) || ((uintptr_t)src & 15) || ((uintptr_t)dst & 15))
+    return MI_TRANSDUCER_INVALID_VALUE;
+  const size_t nvec = bytes / 16;
+  size_t blocks = (nvec + 255) / 256;
+  if (blocks > 256 * 32) blocks = 256 * 32;
+  hipLaunchKernelGGL(copy_probe_kernel, dim3((unsigned)blocks), dim3(256), 0, (hipStream_t)stream, (const uint4*)src,
+                     (uint4*)dst, nvec);
   return launch_status();
 }
 
