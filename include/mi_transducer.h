@@ -69,21 +69,23 @@ int mi_rnnt_forward(const void* acts, int act_dtype, const int64_t* labels, cons
  * gradient of costs[b] w.r.t. the logits for valid cells, FastEmit and clamp folded
  * in (compute_grad_kernel, gpu_rnnt_kernel.py:272-407), zeros for padded cells
  * (replaces zeros_like + `grads *= 0`, rnnt_pytorch.py:58, gpu_rnnt.py:156).
- * grad_scale (nullable, float32 [B]) multiplies utterance b's gradient after the
- * clamp: it folds the autograd backward `grads.mul_(grad_output)` (rnnt_pytorch.py:88-92)
- * and the 'mean' reduction's 1/B (rnnt_pytorch.py:77-81) into the same pass.
+ * Utterance b's gradient is multiplied, after the clamp, by
+ *     (grad_scale ? grad_scale[b * grad_scale_stride] : 1) * grad_mul
+ * which folds the autograd backward `grads.mul_(grad_output)` (rnnt_pytorch.py:88-92; a
+ * broadcast grad_output is stride 0) and the 'mean' reduction's 1/B (rnnt_pytorch.py:77-81)
+ * into the same pass.  grad_scale: device float32, nullable; grad_scale_stride >= 0 in elements.
  * Must follow mi_rnnt_forward(with_betas != 0) on the same workspace and inputs. */
 int mi_rnnt_backward(const void* acts, int act_dtype, const int64_t* labels, const int64_t* act_lens,
-                     const int64_t* label_lens, void* grads, const float* grad_scale, int B, int T, int U, int V,
-                     int blank, float fastemit_lambda, float clamp, void* workspace, size_t workspace_bytes,
-                     void* stream);
+                     const int64_t* label_lens, void* grads, const float* grad_scale, int grad_scale_stride,
+                     float grad_mul, int B, int T, int U, int V, int blank, float fastemit_lambda, float clamp,
+                     void* workspace, size_t workspace_bytes, void* stream);
 
 /* rnnt_loss_gpu in one call (rnnt.py:138-236 -> GPURNNT.cost_and_grad / score_forward,
  * gpu_rnnt.py:125-265): grads == NULL means forward only. */
 int mi_rnnt_loss(const void* acts, int act_dtype, const int64_t* labels, const int64_t* act_lens,
-                 const int64_t* label_lens, float* costs, void* grads, const float* grad_scale, int B, int T, int U,
-                 int V, int blank, float fastemit_lambda, float clamp, void* workspace, size_t workspace_bytes,
-                 void* stream);
+                 const int64_t* label_lens, float* costs, void* grads, const float* grad_scale,
+                 int grad_scale_stride, float grad_mul, int B, int T, int U, int V, int blank, float fastemit_lambda,
+                 float clamp, void* workspace, size_t workspace_bytes, void* stream);
 
 /* TDT.  acts is the COMBINED tensor [B,T,U,V+D]: V token logits (blank included)
  * followed by D duration logits, exactly what TDTLossNumba.forward receives
@@ -102,14 +104,16 @@ int mi_tdt_forward(const void* acts, int act_dtype, const int64_t* labels, const
                    int with_betas, void* workspace, size_t workspace_bytes, void* stream);
 
 int mi_tdt_backward(const void* acts, int act_dtype, const int64_t* labels, const int64_t* act_lens,
-                    const int64_t* label_lens, void* grads, const float* grad_scale, int B, int T, int U, int V, int D,
-                    const int32_t* durations_host, int blank, float fastemit_lambda, float clamp, float sigma,
-                    int use_plain_rnnt, void* workspace, size_t workspace_bytes, void* stream);
+                    const int64_t* label_lens, void* grads, const float* grad_scale, int grad_scale_stride,
+                    float grad_mul, int B, int T, int U, int V, int D, const int32_t* durations_host, int blank,
+                    float fastemit_lambda, float clamp, float sigma, int use_plain_rnnt, void* workspace,
+                    size_t workspace_bytes, void* stream);
 
 int mi_tdt_loss(const void* acts, int act_dtype, const int64_t* labels, const int64_t* act_lens,
-                const int64_t* label_lens, float* costs, void* grads, const float* grad_scale, int B, int T, int U,
-                int V, int D, const int32_t* durations_host, int blank, float fastemit_lambda, float clamp, float sigma,
-                int use_plain_rnnt, void* workspace, size_t workspace_bytes, void* stream);
+                const int64_t* label_lens, float* costs, void* grads, const float* grad_scale, int grad_scale_stride,
+                float grad_mul, int B, int T, int U, int V, int D, const int32_t* durations_host, int blank,
+                float fastemit_lambda, float clamp, float sigma, int use_plain_rnnt, void* workspace,
+                size_t workspace_bytes, void* stream);
 
 /* Stage-level read-out for kernel parity tests (the reference tests launch each
  * kernel on its own, tests/collections/asr/numba/rnnt_loss/utils/test_gpu_rnnt_kernel.py):

@@ -409,6 +409,15 @@ __device__ __forceinline__ double lse_h(double a, double b) {
   return (n == -INFINITY) ? m : r;
 }
 
+// The RNNT recursion keeps "log 0" as a large finite number instead of -inf: sums stay finite
+// (arc values are forced finite too), so the two-operand log-sum-exp needs no special cases.
+constexpr double kLogZero = -1.0e300;
+__device__ __forceinline__ double lse_fin(double a, double b) {
+  const double m = fmax(a, b);
+  const float d = -fabsf((float)(a - b));  // -inf when one operand is log 0: the correction vanishes
+  return m + (double)(__builtin_amdgcn_logf(1.0f + fast_exp2(d * kLog2e)) * 0.6931471805599453f);
+}
+
 // value of the lane below / above (wave shift by one lane through DPP, no LDS round trip);
 // lane 0 / lane 63 receives `fill`
 __device__ __forceinline__ double from_lane_below(double v, double fill) {
@@ -472,9 +481,9 @@ __device__ __forceinline__ float finite_arc(float x) { return fminf(fmaxf(x, -3.
 //   alpha (gpu_rnnt_kernel.py:73-172): every cell pushes e = alpha + lp_label to its right
 //   neighbour and s = alpha + lp_blank to the cell below; the next diagonal is lse(e_in, s_in).
 //   beta  (gpu_rnnt_kernel.py:175-269): pulled from the diagonal above.
-// No boundary tests in the loop: everything starts at -inf, the only finite source is
+// No boundary tests in the loop: everything starts at log 0 (kLogZero), the only finite source is
 // alpha(0,0) = 0 (resp. the corner beta(Tb-1,Ub-1) = lp_blank), and values only flow right/down
-// (resp. left/up), so cells outside the lattice either stay -inf (where they could feed a
+// (resp. left/up), so cells outside the lattice either stay at log 0 (where they could feed a
 // valid cell) or hold junk that no valid cell ever reads.  Every lane stores its K values of
 // every diagonal: the skewed rows are 64*K wide.
 // The arc log-probs of P diagonals are fetched into registers while the previous P
@@ -497,7 +506,7 @@ __global__ __launch_bounds__(64) void rnnt_lattice_kernel(const float* __restric
   const int nd = Tb + Ub - 1;
   const size_t row_pitch = (size_t)A * Us;
   const float* arcs_b = arcs + (size_t)b * ND * row_pitch + u0;
-  const double NINF = -INFINITY;
+  const double NINF = kLogZero;
 
   // rows [n, n + step*P) of the blank and label planes, this lane's K columns (rows clamped into
   // the utterance so that the loads never depend on a branch)
@@ -517,12 +526,12 @@ __global__ __launch_bounds__(64) void rnnt_lattice_kernel(const float* __restric
     double e[K], s[K];
 #pragma unroll
     for (int k = 0; k < K; ++k) e[k] = s[k] = NINF;
-    if (lane == 0) s[0] = 0.0;  // makes alpha(0,0) = lse(-inf, 0) = 0
+    if (lane == 0) s[0] = 0.0;  // makes alpha(0,0) = lse(log 0, 0) = 0
     auto step_fn = [&](int n, const float* bk, const float* lb) {
       const double left = from_lane_below(e[K - 1], NINF);
       double a[K];
 #pragma unroll
-      for (int k = 0; k < K; ++k) a[k] = lse_h(k == 0 ? left : e[k - 1], s[k]);
+      for (int k = 0; k < K; ++k) a[k] = lse_fin(k == 0 ? left : e[k - 1], s[k]);
       store_k<K>(out + (size_t)n * Us, a);
 #pragma unroll
       for (int k = 0; k < K; ++k) {
@@ -574,7 +583,7 @@ __global__ __launch_bounds__(64) void rnnt_lattice_kernel(const float* __restric
 #pragma unroll
       for (int k = 0; k < K; ++k) {
         const double rgt = (k == K - 1) ? right : bt[k + 1];
-        nv[k] = lse_h(rgt + (double)finite_arc(lb[k]), bt[k] + (double)finite_arc(bk[k]));
+        nv[k] = lse_fin(rgt + (double)finite_arc(lb[k]), bt[k] + (double)finite_arc(bk[k]));
       }
       store_k<K>(out + (size_t)n * Us, nv);
 #pragma unroll
@@ -744,29 +753,88 @@ __global__ __launch_bounds__(64) void tdt_lattice_kernel(const float* __restrict
 //                label id (-1 none, -2 padded cell), -, -, dlogit_0 .. dlogit_{D-1} }
 // where G_blank / G_label are the finished gradient entries of the two special logits.
 // ----------------------------------------------------------------------------------------
-__device__ __forceinline__ void write_coef(float* c, float dn, float W, float PB, float PL, float lpb, float lpl,
-                                           int lab, int blank, float clamp, float scale) {
-  float gb = expf(lpb) * W - PB;
-  float gl = lab >= 0 ? expf(lpl) * W - PL : 0.f;
-  if (lab == blank) gb = gl = expf(lpb) * W - PB - PL;
+// what the gradient pass needs to derive a row's coefficients itself (RNNT, fused path)
+struct LatticeView {
+  const float* denom;
+  const float* arcs;
+  const double* alphas;
+  const double* betas;
+  const double* ll;
+  const int64_t* labels;
+  const float* grad_scale;
+  int grad_scale_stride;
+  float grad_mul;
+  int ND, Us, A;
+  float lambda, clamp;
+};
+
+struct RowCoef {
+  float dl2;  // denom * log2(e)
+  float W;    // occupancy weight * scale
+  float cb;   // clamp bound * |scale| (inf = no clamp)
+  float gB;   // finished gradient entry of the blank logit
+  float gL;   // finished gradient entry of the label logit
+  int lab;    // label id, -1 if the cell has no label arc
+};
+
+__device__ __forceinline__ RowCoef make_coef(float dn, float W, float PB, float PL, float lpb, float lpl, int lab,
+                                             int blank, float clamp, float scale) {
+  float gb = __expf(lpb) * W - PB;
+  float gl = lab >= 0 ? __expf(lpl) * W - PL : 0.f;
+  if (lab == blank) gb = gl = __expf(lpb) * W - PB - PL;
   if (clamp > 0.f) {
     gb = clamp_sym(gb, clamp);
     gl = clamp_sym(gl, clamp);
   }
-  c[0] = dn * kLog2e;
-  c[1] = W * scale;
-  c[2] = clamp > 0.f ? clamp * fabsf(scale) : INFINITY;
-  c[3] = gb * scale;
-  c[4] = gl * scale;
-  c[5] = __int_as_float(lab);
+  RowCoef c;
+  c.dl2 = dn * kLog2e;
+  c.W = W * scale;
+  c.cb = clamp > 0.f ? clamp * fabsf(scale) : INFINITY;
+  c.gB = gb * scale;
+  c.gL = gl * scale;
+  c.lab = lab;
+  return c;
+}
+
+__device__ __forceinline__ void write_coef(float* out, const RowCoef& c) {
+  out[0] = c.dl2;
+  out[1] = c.W;
+  out[2] = c.cb;
+  out[3] = c.gB;
+  out[4] = c.gL;
+  out[5] = __int_as_float(c.lab);
+}
+
+// the RNNT coefficients of cell (b,t,u) from the lattice state (gpu_rnnt_kernel.py:340-403)
+__device__ __forceinline__ RowCoef rnnt_coef(const float* __restrict__ denom, const float* __restrict__ arcs,
+                                             const double* __restrict__ alphas, const double* __restrict__ betas,
+                                             const double* __restrict__ ll, const int64_t* __restrict__ labels,
+                                             float scale, int b, int t, int u, int Tb, int Ub, int T, int U, int V,
+                                             int blank, int ND, int Us, int A, float lambda, float clamp) {
+  const size_t row = (size_t)(b * ND + t + u);
+  const size_t sk = row * Us + u;
+  const double a = alphas[sk], bb = betas[sk], L = ll[2 * b];
+  const float lpb = arcs[row * A * Us + u];
+  const float lpl = arcs[row * A * Us + Us + u];
+  const int lab = (u < Ub - 1) ? clampi(labels[(size_t)b * (U - 1) + u], 0, V - 1) : -1;
+  // the clamped indices keep the loads unconditional; their values are dropped by the selects below
+  const double b_down = betas[sk + (t < Tb - 1 ? Us : 0)];         // beta(t+1,u): next diagonal, same column
+  const double b_right = betas[sk + (lab >= 0 ? Us + 1 : 0)];      // beta(t,u+1)
+  const float gamma = __expf((float)(a + bb - L));
+  float pb = 0.f, pl = 0.f;
+  if (t < Tb - 1) pb = __expf((float)(a + b_down - L + (double)lpb));
+  else if (u == Ub - 1) pb = __expf((float)(a - L + (double)lpb));
+  if (lab >= 0) pl = __expf((float)(a + b_right - L + (double)lpl));
+  const float dn = denom[((size_t)b * T + t) * U + u];
+  return make_coef(dn, gamma + lambda * pl, pb, (1.f + lambda) * pl, lpb, lpl, lab, blank, clamp, scale);
 }
 
 __global__ __launch_bounds__(256) void rnnt_cell_kernel(
     const float* __restrict__ denom, const float* __restrict__ arcs, const double* __restrict__ alphas,
     const double* __restrict__ betas, const double* __restrict__ ll, const int64_t* __restrict__ labels,
     const int64_t* __restrict__ act_lens, const int64_t* __restrict__ label_lens, const float* __restrict__ grad_scale,
-    float* __restrict__ coef, int T, int U, int V, int blank, int ND, int Us, int A, int CS, float lambda, float clamp,
-    long long cells) {
+    int grad_scale_stride, float grad_mul, float* __restrict__ coef, int T, int U, int V, int blank, int ND, int Us,
+    int A, int CS, float lambda, float clamp, long long cells) {
   const long long c = (long long)blockIdx.x * blockDim.x + threadIdx.x;
   if (c >= cells) return;
   const int u = (int)(c % U);
@@ -780,29 +848,17 @@ __global__ __launch_bounds__(256) void rnnt_cell_kernel(
     out[5] = __int_as_float(-2);
     return;
   }
-  const size_t row = (size_t)(b * ND + t + u);
-  const size_t sk = row * Us + u;
-  const double a = alphas[sk], bb = betas[sk], L = ll[2 * b];
-  const float lpb = arcs[row * A * Us + u];
-  const float lpl = arcs[row * A * Us + Us + u];
-  const int lab = (u < Ub - 1) ? clampi(labels[(size_t)b * (U - 1) + u], 0, V - 1) : -1;
-  const float gamma = expf((float)(a + bb - L));
-  float pb = 0.f, pl = 0.f;
-  if (t < Tb - 1)
-    pb = expf((float)(a + betas[sk + Us] - L + (double)lpb));  // beta(t+1,u): next diagonal, same column
-  else if (u == Ub - 1)
-    pb = expf((float)(a - L + (double)lpb));
-  if (lab >= 0) pl = expf((float)(a + betas[sk + Us + 1] - L + (double)lpl));  // beta(t,u+1)
-  const float scale = grad_scale ? grad_scale[b] : 1.f;
-  write_coef(out, denom[c], gamma + lambda * pl, pb, (1.f + lambda) * pl, lpb, lpl, lab, blank, clamp, scale);
+  const float scale = (grad_scale ? grad_scale[(size_t)b * grad_scale_stride] : 1.f) * grad_mul;
+  write_coef(out, rnnt_coef(denom, arcs, alphas, betas, ll, labels, scale, b, t, u, Tb, Ub, T, U, V, blank, ND, Us, A,
+                            lambda, clamp));
 }
 
 __global__ __launch_bounds__(256) void tdt_cell_kernel(
     const float* __restrict__ denom, const float* __restrict__ arcs, const double* __restrict__ alphas,
     const double* __restrict__ betas, const double* __restrict__ ll, const int64_t* __restrict__ labels,
     const int64_t* __restrict__ act_lens, const int64_t* __restrict__ label_lens, const float* __restrict__ grad_scale,
-    float* __restrict__ coef, int T, int U, int V, int blank, int ND, int Us, int A, int CS, float lambda, float clamp,
-    long long cells, TdtParams prm) {
+    int grad_scale_stride, float grad_mul, float* __restrict__ coef, int T, int U, int V, int blank, int ND, int Us,
+    int A, int CS, float lambda, float clamp, long long cells, TdtParams prm) {
   const long long c = (long long)blockIdx.x * blockDim.x + threadIdx.x;
   if (c >= cells) return;
   const int u = (int)(c % U);
@@ -824,7 +880,7 @@ __global__ __launch_bounds__(256) void tdt_cell_kernel(
   const float* rp = arcs + row * A * Us + u;
   const float lpb = rp[0], lpl = rp[Us];
   const int lab = (u < Ub - 1) ? clampi(labels[(size_t)b * (U - 1) + u], 0, V - 1) : -1;
-  const float scale = grad_scale ? grad_scale[b] : 1.f;
+  const float scale = (grad_scale ? grad_scale[(size_t)b * grad_scale_stride] : 1.f) * grad_mul;
   const float gamma = expf((float)(a + bb - L));
   float pb = 0.f, pl = 0.f;
   float arc_post[MI_TRANSDUCER_MAX_DURATIONS], q[MI_TRANSDUCER_MAX_DURATIONS];
@@ -850,7 +906,7 @@ __global__ __launch_bounds__(256) void tdt_cell_kernel(
   const float tot = pl + pb;
 #pragma unroll 1
   for (int i = 0; i < D; ++i) out[kCoefBase + i] = (q[i] * tot - arc_post[i]) * scale;
-  write_coef(out, denom[c], gamma + lambda * pl, pb, (1.f + lambda) * pl, lpb, lpl, lab, blank, clamp, scale);
+  write_coef(out, make_coef(denom[c], gamma + lambda * pl, pb, (1.f + lambda) * pl, lpb, lpl, lab, blank, clamp, scale));
 }
 
 // ----------------------------------------------------------------------------------------
@@ -1140,9 +1196,11 @@ __global__ __launch_bounds__(256) void denom_rows_kernel(
   }
 }
 
-template <int DT, int R>
+// FUSED (RNNT): the row's coefficients are derived here from the lattice state, one wave-uniform
+// evaluation per row, instead of being read from the coefficient buffer a cell kernel filled.
+template <int DT, int R, bool FUSED>
 __global__ __launch_bounds__(256) void grad_rows_kernel(const void* __restrict__ acts, void* __restrict__ grads,
-                                                        const float* __restrict__ coef,
+                                                        const float* __restrict__ coef, LatticeView lv,
                                                         const int64_t* __restrict__ act_lens,
                                                         const int64_t* __restrict__ label_lens, int T, int U, int V,
                                                         int D, int blank, int CS, int zero_durations, int nchunks,
@@ -1169,20 +1227,19 @@ __global__ __launch_bounds__(256) void grad_rows_kernel(const void* __restrict__
   zero_elems<DT>(grads, (cell0 + z0) * VD, (cell0 + c1) * VD);
   const int u_begin = c0 + wave;
   if (u_begin >= z0) return;
+  float scale = 1.f;
+  if constexpr (FUSED) scale = (lv.grad_scale ? lv.grad_scale[(size_t)b * lv.grad_scale_stride] : 1.f) * lv.grad_mul;
 
   struct Row {
     uint4 raw[R];
-    float4 ca;
-    float2 cb;
+    RowCoef c;
     float xe, gd;
     int mis;
   };
   // head, tail and duration entries of a row: one element per lane
   auto extra_index = [&](const RowSplit<DT>& sp) {
-    int v = -1;
-    if (lane < sp.hc) v = lane;
-    else if (lane >= VEC && lane < VEC + sp.tc) v = sp.tail0() + lane - VEC;
-    else if (lane >= 2 * VEC && lane < 2 * VEC + D) v = V + lane - 2 * VEC;
+    int v = sp.extra_token(lane);
+    if (lane >= 2 * VEC && lane < 2 * VEC + D) v = V + lane - 2 * VEC;
     return v;
   };
   auto fetch = [&](int uu, Row& d) {
@@ -1193,18 +1250,26 @@ __global__ __launch_bounds__(256) void grad_rows_kernel(const void* __restrict__
     // unconditional loads, as in the denominator pass
 #pragma unroll
     for (int k = 0; k < R; ++k) d.raw[k] = load_stream<MI_NT_K4 != 0>(w.vp + sp.body_vector(lane + 64 * k));
-    const float* c = coef + (cell0 + uu) * CS;
-    d.ca = *(const float4*)c;        // denom*log2e, W*scale, clamp bound, G_blank
-    d.cb = *(const float2*)(c + 4);  // G_label, label id
     const int v = extra_index(sp);
     d.xe = Elem<DT>::load1(acts, e0 + ((v >= 0 && v < V) ? v : blank));
-    d.gd = c[v >= V ? kCoefBase + v - V : 0];
+    if constexpr (FUSED) {
+      d.c = rnnt_coef(lv.denom, lv.arcs, lv.alphas, lv.betas, lv.ll, lv.labels, scale, b, t, uu, Tb, Ub, T, U, V, blank,
+                      lv.ND, lv.Us, lv.A, lv.lambda, lv.clamp);
+      d.gd = 0.f;
+    } else {
+      const float* c = coef + (cell0 + uu) * CS;
+      const float4 ca = *(const float4*)c;        // denom*log2e, W*scale, clamp bound, G_blank
+      const float2 cb = *(const float2*)(c + 4);  // G_label, label id
+      d.c.dl2 = ca.x; d.c.W = ca.y; d.c.cb = ca.z; d.c.gB = ca.w; d.c.gL = cb.x;
+      d.c.lab = __float_as_int(cb.y);
+      d.gd = c[v >= V ? kCoefBase + v - V : 0];
+    }
   };
   auto emit = [&](int uu, const Row& d) {
     const size_t e0 = (cell0 + uu) * VD;
     const RowSplit<DT> sp(d.mis, V);
-    const float dl2 = d.ca.x, W = d.ca.y, cb = d.ca.z, gB = d.ca.w, gL = d.cb.x;
-    const int lab = __float_as_int(d.cb.y);
+    const float dl2 = d.c.dl2, W = d.c.W, cb = d.c.cb, gB = d.c.gB, gL = d.c.gL;
+    const int lab = d.c.lab;
     const bool clamp_on = cb < INFINITY;
     char* grow = (char*)grads + e0 * Elem<DT>::BYTES;  // same 16-byte phase as the acts row
     uint4* gvp = (uint4*)(grow - d.mis * Elem<DT>::BYTES) + sp.jb0 + lane;
@@ -1430,6 +1495,11 @@ inline int rows_R(const Common& c) {
     if (nb <= 64 * r) return r;
   return 0;
 }
+// the row kernels store gradient vectors at the 16-byte phase of the logits row
+inline int grad_rows_R(const Common& c, const void* grads) {
+  const bool same_phase = (((uintptr_t)c.acts ^ (uintptr_t)grads) & 15) == 0;
+  return same_phase ? rows_R(c) : 0;
+}
 inline int chunks_of(const Common& c) { return (c.U + kChunkRows - 1) / kChunkRows; }
 inline int chunk_blocks(const Common& c) { return chunks_of(c) * c.B * c.T; }
 // rounded up to whole turns of the XCD permutation
@@ -1524,17 +1594,44 @@ int run_tdt_lattice(const Common& c, float* costs, float lambda, int with_betas,
   return launch_status();
 }
 
-int run_grad_stream(const Common& c, void* grads, int zero_durations) {
+struct ScaleArg {
+  const float* ptr;
+  int stride;
+  float mul;
+};
+
+// fused != 0: RNNT rows derive their coefficients from the lattice state inside the pass
+// (needs no cell kernel); only the register-resident row kernels can do that
+int run_grad_stream(const Common& c, void* grads, int zero_durations, bool fused, const ScaleArg& sc, float lambda,
+                    float clamp) {
   const Layout& L = c.L;
   const float* coef = (const float*)(c.ws + L.off_coef);
   const RowGrid g = row_grid(c);
-  // the row kernels store gradient vectors at the 16-byte phase of the logits row
-  const bool same_phase = (((uintptr_t)c.acts ^ (uintptr_t)grads) & 15) == 0;
-  const int R = same_phase ? rows_R(c) : 0;
+  LatticeView lv;
+  lv.denom = (const float*)(c.ws + L.off_denom);
+  lv.arcs = (const float*)(c.ws + L.off_arcs);
+  lv.alphas = (const double*)(c.ws + L.off_alphas);
+  lv.betas = (const double*)(c.ws + L.off_betas);
+  lv.ll = (const double*)(c.ws + L.off_ll);
+  lv.labels = c.labels;
+  lv.grad_scale = sc.ptr;
+  lv.grad_scale_stride = sc.stride;
+  lv.grad_mul = sc.mul;
+  lv.ND = L.ND; lv.Us = L.Us; lv.A = L.A;
+  lv.lambda = lambda; lv.clamp = clamp;
+  const int R = grad_rows_R(c, grads);
   ProfScope prof(MI_PROFILE_GRAD, c.stream);
 #define LAUNCH_GRAD_ROWS(DT, RR)                                                                                    \
-  hipLaunchKernelGGL((grad_rows_kernel<DT, RR>), chunk_grid(c), dim3(256), 0, c.stream, c.acts, grads, coef,         \
-                     c.act_lens, c.label_lens, c.T, c.U, c.V, c.D, c.blank, L.CS, zero_durations, chunks_of(c), chunk_blocks(c))
+  do {                                                                                                              \
+    if (fused)                                                                                                      \
+      hipLaunchKernelGGL((grad_rows_kernel<DT, RR, true>), chunk_grid(c), dim3(256), 0, c.stream, c.acts, grads,     \
+                         coef, lv, c.act_lens, c.label_lens, c.T, c.U, c.V, c.D, c.blank, L.CS, zero_durations,      \
+                         chunks_of(c), chunk_blocks(c));                                                            \
+    else                                                                                                            \
+      hipLaunchKernelGGL((grad_rows_kernel<DT, RR, false>), chunk_grid(c), dim3(256), 0, c.stream, c.acts, grads,    \
+                         coef, lv, c.act_lens, c.label_lens, c.T, c.U, c.V, c.D, c.blank, L.CS, zero_durations,      \
+                         chunks_of(c), chunk_blocks(c));                                                            \
+  } while (0)
 #define LAUNCH_GRAD(DT)                                                                                             \
   do {                                                                                                              \
     switch (R) {                                                                                                    \
@@ -1555,7 +1652,7 @@ int run_grad_stream(const Common& c, void* grads, int zero_durations) {
   return launch_status();
 }
 
-int run_rnnt_cells(const Common& c, const float* grad_scale, float lambda, float clamp) {
+int run_rnnt_cells(const Common& c, const ScaleArg& sc, float lambda, float clamp) {
   const Layout& L = c.L;
   const long long cells = (long long)c.B * c.T * c.U;
   const unsigned grid = (unsigned)((cells + 255) / 256);
@@ -1563,12 +1660,12 @@ int run_rnnt_cells(const Common& c, const float* grad_scale, float lambda, float
   hipLaunchKernelGGL(rnnt_cell_kernel, dim3(grid), dim3(256), 0, c.stream, (const float*)(c.ws + L.off_denom),
                      (const float*)(c.ws + L.off_arcs), (const double*)(c.ws + L.off_alphas),
                      (const double*)(c.ws + L.off_betas), (const double*)(c.ws + L.off_ll), c.labels, c.act_lens,
-                     c.label_lens, grad_scale, (float*)(c.ws + L.off_coef), c.T, c.U, c.V, c.blank, L.ND, L.Us, L.A,
-                     L.CS, lambda, clamp, cells);
+                     c.label_lens, sc.ptr, sc.stride, sc.mul, (float*)(c.ws + L.off_coef), c.T, c.U, c.V, c.blank, L.ND,
+                     L.Us, L.A, L.CS, lambda, clamp, cells);
   return launch_status();
 }
 
-int run_tdt_cells(const Common& c, const float* grad_scale, float lambda, float clamp, const TdtParams& prm) {
+int run_tdt_cells(const Common& c, const ScaleArg& sc, float lambda, float clamp, const TdtParams& prm) {
   const Layout& L = c.L;
   const long long cells = (long long)c.B * c.T * c.U;
   const unsigned grid = (unsigned)((cells + 255) / 256);
@@ -1576,8 +1673,8 @@ int run_tdt_cells(const Common& c, const float* grad_scale, float lambda, float 
   hipLaunchKernelGGL(tdt_cell_kernel, dim3(grid), dim3(256), 0, c.stream, (const float*)(c.ws + L.off_denom),
                      (const float*)(c.ws + L.off_arcs), (const double*)(c.ws + L.off_alphas),
                      (const double*)(c.ws + L.off_betas), (const double*)(c.ws + L.off_ll), c.labels, c.act_lens,
-                     c.label_lens, grad_scale, (float*)(c.ws + L.off_coef), c.T, c.U, c.V, c.blank, L.ND, L.Us, L.A,
-                     L.CS, lambda, clamp, cells, prm);
+                     c.label_lens, sc.ptr, sc.stride, sc.mul, (float*)(c.ws + L.off_coef), c.T, c.U, c.V, c.blank, L.ND,
+                     L.Us, L.A, L.CS, lambda, clamp, cells, prm);
   return launch_status();
 }
 
@@ -1588,7 +1685,7 @@ int run_tdt_cells(const Common& c, const float* grad_scale, float lambda, float 
 // ----------------------------------------------------------------------------------------
 extern "C" {
 
-int mi_transducer_abi_version(void) { return 1; }
+int mi_transducer_abi_version(void) { return 2; }
 
 int mi_transducer_workspace_bytes(int B, int T, int U, int D, size_t* out_bytes) {
   Layout L;
@@ -1610,27 +1707,29 @@ int mi_rnnt_forward(const void* acts, int act_dtype, const int64_t* labels, cons
 }
 
 int mi_rnnt_backward(const void* acts, int act_dtype, const int64_t* labels, const int64_t* act_lens,
-                     const int64_t* label_lens, void* grads, const float* grad_scale, int B, int T, int U, int V,
-                     int blank, float fastemit_lambda, float clamp, void* workspace, size_t workspace_bytes,
-                     void* stream) {
+                     const int64_t* label_lens, void* grads, const float* grad_scale, int grad_scale_stride,
+                     float grad_mul, int B, int T, int U, int V, int blank, float fastemit_lambda, float clamp,
+                     void* workspace, size_t workspace_bytes, void* stream) {
   Common c;
-  if (!grads || clamp < 0.f) return MI_TRANSDUCER_INVALID_VALUE;
+  if (!grads || clamp < 0.f || grad_scale_stride < 0) return MI_TRANSDUCER_INVALID_VALUE;
   int st = check_common(acts, act_dtype, labels, act_lens, label_lens, B, T, U, V, 0, blank, workspace,
                         workspace_bytes, stream, &c);
   if (st) return st;
-  if ((st = run_rnnt_cells(c, grad_scale, fastemit_lambda, clamp))) return st;
-  return run_grad_stream(c, grads, 0);
+  const ScaleArg sc = {grad_scale, grad_scale_stride, grad_mul};
+  const bool fused = grad_rows_R(c, grads) != 0;
+  if (!fused && (st = run_rnnt_cells(c, sc, fastemit_lambda, clamp))) return st;
+  return run_grad_stream(c, grads, 0, fused, sc, fastemit_lambda, clamp);
 }
 
 int mi_rnnt_loss(const void* acts, int act_dtype, const int64_t* labels, const int64_t* act_lens,
-                 const int64_t* label_lens, float* costs, void* grads, const float* grad_scale, int B, int T, int U,
-                 int V, int blank, float fastemit_lambda, float clamp, void* workspace, size_t workspace_bytes,
-                 void* stream) {
+                 const int64_t* label_lens, float* costs, void* grads, const float* grad_scale,
+                 int grad_scale_stride, float grad_mul, int B, int T, int U, int V, int blank, float fastemit_lambda,
+                 float clamp, void* workspace, size_t workspace_bytes, void* stream) {
   int st = mi_rnnt_forward(acts, act_dtype, labels, act_lens, label_lens, costs, B, T, U, V, blank, fastemit_lambda,
                            grads != nullptr, workspace, workspace_bytes, stream);
   if (st || !grads) return st;
-  return mi_rnnt_backward(acts, act_dtype, labels, act_lens, label_lens, grads, grad_scale, B, T, U, V, blank,
-                          fastemit_lambda, clamp, workspace, workspace_bytes, stream);
+  return mi_rnnt_backward(acts, act_dtype, labels, act_lens, label_lens, grads, grad_scale, grad_scale_stride,
+                          grad_mul, B, T, U, V, blank, fastemit_lambda, clamp, workspace, workspace_bytes, stream);
 }
 
 int mi_tdt_forward(const void* acts, int act_dtype, const int64_t* labels, const int64_t* act_lens,
@@ -1652,35 +1751,39 @@ int mi_tdt_forward(const void* acts, int act_dtype, const int64_t* labels, const
 }
 
 int mi_tdt_backward(const void* acts, int act_dtype, const int64_t* labels, const int64_t* act_lens,
-                    const int64_t* label_lens, void* grads, const float* grad_scale, int B, int T, int U, int V, int D,
-                    const int32_t* durations_host, int blank, float fastemit_lambda, float clamp, float sigma,
-                    int use_plain_rnnt, void* workspace, size_t workspace_bytes, void* stream) {
+                    const int64_t* label_lens, void* grads, const float* grad_scale, int grad_scale_stride,
+                    float grad_mul, int B, int T, int U, int V, int D, const int32_t* durations_host, int blank,
+                    float fastemit_lambda, float clamp, float sigma, int use_plain_rnnt, void* workspace,
+                    size_t workspace_bytes, void* stream) {
   Common c;
   TdtParams prm;
-  if (!grads || clamp < 0.f) return MI_TRANSDUCER_INVALID_VALUE;
+  if (!grads || clamp < 0.f || grad_scale_stride < 0) return MI_TRANSDUCER_INVALID_VALUE;
   int st = make_tdt_params(D, durations_host, sigma, &prm);
   if (st) return st;
   st = check_common(acts, act_dtype, labels, act_lens, label_lens, B, T, U, V, D, blank, workspace, workspace_bytes,
                     stream, &c);
   if (st) return st;
+  const ScaleArg sc = {grad_scale, grad_scale_stride, grad_mul};
   if (use_plain_rnnt) {  // gpu_rnnt.py:646-682: token gradient from the RNNT kernel, duration gradient stays zero
-    if ((st = run_rnnt_cells(c, grad_scale, fastemit_lambda, clamp))) return st;
-    return run_grad_stream(c, grads, 1);
+    const bool fused = grad_rows_R(c, grads) != 0;
+    if (!fused && (st = run_rnnt_cells(c, sc, fastemit_lambda, clamp))) return st;
+    return run_grad_stream(c, grads, 1, fused, sc, fastemit_lambda, clamp);
   }
-  if ((st = run_tdt_cells(c, grad_scale, fastemit_lambda, clamp, prm))) return st;
-  return run_grad_stream(c, grads, 0);
+  if ((st = run_tdt_cells(c, sc, fastemit_lambda, clamp, prm))) return st;
+  return run_grad_stream(c, grads, 0, false, sc, fastemit_lambda, clamp);
 }
 
 int mi_tdt_loss(const void* acts, int act_dtype, const int64_t* labels, const int64_t* act_lens,
-                const int64_t* label_lens, float* costs, void* grads, const float* grad_scale, int B, int T, int U,
-                int V, int D, const int32_t* durations_host, int blank, float fastemit_lambda, float clamp, float sigma,
-                int use_plain_rnnt, void* workspace, size_t workspace_bytes, void* stream) {
+                const int64_t* label_lens, float* costs, void* grads, const float* grad_scale, int grad_scale_stride,
+                float grad_mul, int B, int T, int U, int V, int D, const int32_t* durations_host, int blank,
+                float fastemit_lambda, float clamp, float sigma, int use_plain_rnnt, void* workspace,
+                size_t workspace_bytes, void* stream) {
   int st = mi_tdt_forward(acts, act_dtype, labels, act_lens, label_lens, costs, B, T, U, V, D, durations_host, blank,
                           fastemit_lambda, sigma, use_plain_rnnt, grads != nullptr, workspace, workspace_bytes, stream);
   if (st || !grads) return st;
-  return mi_tdt_backward(acts, act_dtype, labels, act_lens, label_lens, grads, grad_scale, B, T, U, V, D,
-                         durations_host, blank, fastemit_lambda, clamp, sigma, use_plain_rnnt, workspace,
-                         workspace_bytes, stream);
+  return mi_tdt_backward(acts, act_dtype, labels, act_lens, label_lens, grads, grad_scale, grad_scale_stride, grad_mul,
+                         B, T, U, V, D, durations_host, blank, fastemit_lambda, clamp, sigma, use_plain_rnnt,
+                         workspace, workspace_bytes, stream);
 }
 
 int mi_transducer_export_lattice(const void* workspace, size_t workspace_bytes, const int64_t* act_lens,

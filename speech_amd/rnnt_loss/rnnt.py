@@ -92,15 +92,18 @@ def rnnt_forward(acts, labels, act_lens, label_lens, costs, blank, fastemit_lamb
 
 
 def rnnt_backward(
-    acts, labels, act_lens, label_lens, grads, grad_scale, blank, fastemit_lambda, clamp, workspace
-):
+    acts, labels, act_lens, label_lens, grads, grad_scale, blank, fastemit_lambda, clamp, workspace,
+    grad_scale_stride=1, grad_mul=1.0,
+):  # fmt: skip
+    """grad_scale: device float32 tensor read as grad_scale[b * grad_scale_stride] (or None); every gradient is
+    additionally multiplied by the host scalar grad_mul."""
     _require_gpu(acts, "rnnt_backward")
     B, T, U, V = acts.shape
     with torch.cuda.device(acts.device):
         status = _native.lib().mi_rnnt_backward(
             _ptr(acts), _dtype_code(acts), _labels_ptr(labels), _ptr(act_lens), _ptr(label_lens), _ptr(grads),
-            _ptr(grad_scale), B, T, U, V, int(blank), float(fastemit_lambda), float(clamp),
-            _ptr(workspace), workspace.numel(), _stream(acts.device),
+            _ptr(grad_scale), int(grad_scale_stride), float(grad_mul), B, T, U, V, int(blank), float(fastemit_lambda),
+            float(clamp), _ptr(workspace), workspace.numel(), _stream(acts.device),
         )  # fmt: skip
     _native.check_status(status, "Could not calculate gradients")
 
@@ -125,7 +128,7 @@ def tdt_forward(
 
 def tdt_backward(
     acts, labels, act_lens, label_lens, grads, grad_scale, blank, durations, fastemit_lambda, clamp, sigma,
-    use_plain_rnnt, workspace,
+    use_plain_rnnt, workspace, grad_scale_stride=1, grad_mul=1.0,
 ):  # fmt: skip
     _require_gpu(acts, "tdt_backward")
     B, T, U, VD = acts.shape
@@ -134,8 +137,9 @@ def tdt_backward(
     with torch.cuda.device(acts.device):
         status = _native.lib().mi_tdt_backward(
             _ptr(acts), _dtype_code(acts), _labels_ptr(labels), _ptr(act_lens), _ptr(label_lens), _ptr(grads),
-            _ptr(grad_scale), B, T, U, VD - D, D, dur_ptr, int(blank), float(fastemit_lambda), float(clamp),
-            float(sigma), int(bool(use_plain_rnnt)), _ptr(workspace), workspace.numel(), _stream(acts.device),
+            _ptr(grad_scale), int(grad_scale_stride), float(grad_mul), B, T, U, VD - D, D, dur_ptr, int(blank),
+            float(fastemit_lambda), float(clamp), float(sigma), int(bool(use_plain_rnnt)), _ptr(workspace),
+            workspace.numel(), _stream(acts.device),
         )  # fmt: skip
     del keep
     _native.check_status(status, "Could not calculate gradients")
@@ -171,7 +175,7 @@ def rnnt_loss_gpu(
     with torch.cuda.device(acts.device):
         status = _native.lib().mi_rnnt_loss(
             _ptr(acts), _dtype_code(acts), _labels_ptr(labels), _ptr(input_lengths), _ptr(label_lengths), _ptr(costs),
-            _ptr(grads), None, B, T, U, V, int(blank_label), float(fastemit_lambda), float(clamp),
+            _ptr(grads), None, 0, 1.0, B, T, U, V, int(blank_label), float(fastemit_lambda), float(clamp),
             _ptr(workspace), workspace.numel(), _stream(acts.device),
         )  # fmt: skip
     _native.check_status(status, "Could not calculate forward scores")
@@ -195,8 +199,9 @@ def tdt_loss_gpu(
     with torch.cuda.device(acts.device):
         status = _native.lib().mi_tdt_loss(
             _ptr(acts), _dtype_code(acts), _labels_ptr(labels), _ptr(input_lengths), _ptr(label_lengths), _ptr(costs),
-            _ptr(grads), None, B, T, U, VD - D, D, dur_ptr, int(blank_label), float(fastemit_lambda), float(clamp),
-            float(sigma), int(bool(use_plain_rnnt)), _ptr(workspace), workspace.numel(), _stream(acts.device),
+            _ptr(grads), None, 0, 1.0, B, T, U, VD - D, D, dur_ptr, int(blank_label), float(fastemit_lambda),
+            float(clamp), float(sigma), int(bool(use_plain_rnnt)), _ptr(workspace), workspace.numel(),
+            _stream(acts.device),
         )  # fmt: skip
     del keep
     _native.check_status(status, "Could not calculate forward scores")

@@ -124,16 +124,21 @@ def _reduce_costs(costs, reduction, batch):
 
 
 def _grad_scale(grad_output, reduction, batch, device):
-    # what the reference applies to its stored gradient: /B for 'mean' in forward
-    # (rnnt_pytorch.py:77-81), then * grad_output broadcast over the batch in backward (:88-92)
-    scale = grad_output.detach().to(device=device, dtype=torch.float32).reshape(-1)
-    if scale.numel() == 1:
-        scale = scale.expand(batch)
-    elif scale.numel() != batch:
-        raise RuntimeError(f"grad_output has {scale.numel()} elements, expected 1 or {batch}")
-    if reduction == 'mean':
-        scale = scale / batch
-    return scale.contiguous()
+    """(tensor, stride, multiplier) such that utterance b's gradient is scaled by
+    tensor[b * stride] * multiplier: what the reference applies to its stored gradient -- 1/B for
+    'mean' in forward (rnnt_pytorch.py:77-81), then grad_output broadcast over the batch in backward
+    (:88-92).  The usual cases (a dense or a broadcast float32 grad_output) need no copy."""
+    mul = 1.0 / batch if reduction == 'mean' else 1.0
+    g = grad_output.detach()
+    if g.dtype != torch.float32 or g.device != device:
+        g = g.to(device=device, dtype=torch.float32)
+    if g.numel() == 1:
+        return g.reshape(1), 0, mul
+    if g.numel() != batch:
+        raise RuntimeError(f"grad_output has {g.numel()} elements, expected 1 or {batch}")
+    if g.dim() != 1:
+        g = g.reshape(batch)
+    return g, g.stride(0), mul
 
 
 class _RNNTNumba(Function):
@@ -167,8 +172,10 @@ class _RNNTNumba(Function):
         acts, labels, act_lens, label_lens, workspace = ctx.saved_tensors
         blank, reduction, fastemit_lambda, clamp = ctx.params
         grads = torch.empty_like(acts)
-        scale = _grad_scale(grad_output, reduction, acts.size(0), acts.device)
-        rnnt.rnnt_backward(acts, labels, act_lens, label_lens, grads, scale, blank, fastemit_lambda, clamp, workspace)
+        scale, stride, mul = _grad_scale(grad_output, reduction, acts.size(0), acts.device)
+        rnnt.rnnt_backward(
+            acts, labels, act_lens, label_lens, grads, scale, blank, fastemit_lambda, clamp, workspace, stride, mul
+        )
         return grads, None, None, None, None, None, None, None
 
 
@@ -215,10 +222,10 @@ class _TDTNumba(Function):
         acts, labels, act_lens, label_lens, workspace = ctx.saved_tensors
         blank, durations, reduction, fastemit_lambda, clamp, sigma, use_plain_rnnt = ctx.params
         grads = torch.empty_like(acts)
-        scale = _grad_scale(grad_output, reduction, acts.size(0), acts.device)
+        scale, stride, mul = _grad_scale(grad_output, reduction, acts.size(0), acts.device)
         rnnt.tdt_backward(
             acts, labels, act_lens, label_lens, grads, scale, blank, durations, fastemit_lambda, clamp, sigma,
-            use_plain_rnnt, workspace,
+            use_plain_rnnt, workspace, stride, mul,
         )  # fmt: skip
         return grads, None, None, None, None, None, None, None, None, None, None
 
