@@ -133,9 +133,11 @@ int mi_transducer_length_maxima(const int64_t* act_lens, const int64_t* label_le
 
 /* ---- benchmark aids (no counterpart in the reference) --------------------------------
  * Per-kernel timing of the launches a harness itself makes: after
- * mi_transducer_profile_enable(n), each of the next n launches of every pipeline kernel is
- * bracketed by a pair of HIP events on its stream (enable creates the events: the one
- * place this library allocates).  mi_transducer_profile_read waits for the recorded
+ * mi_transducer_profile_enable(n, mask), each of the next n launches of every pipeline kernel
+ * whose bit (1 << MI_PROFILE_*) is set in mask is bracketed by a pair of HIP events on its
+ * stream (enable creates the events: the one place this library allocates).  An event pair
+ * costs a few microseconds of queue time, so a harness that also times whole steps should
+ * select only the kernel it needs.  mi_transducer_profile_read waits for the recorded
  * launches of one kernel class, returns their summed duration and count, and resets that
  * class.  Not thread-safe; leave disabled outside benchmarks. */
 #define MI_PROFILE_DENOM 0   /* denom_gather_kernel */
@@ -143,7 +145,7 @@ int mi_transducer_length_maxima(const int64_t* act_lens, const int64_t* label_le
 #define MI_PROFILE_CELL 2    /* rnnt_cell_kernel / tdt_cell_kernel */
 #define MI_PROFILE_GRAD 3    /* grad_stream_kernel */
 #define MI_PROFILE_KERNELS 4
-int mi_transducer_profile_enable(int max_launches);
+int mi_transducer_profile_enable(int max_launches, unsigned kernel_mask);
 int mi_transducer_profile_read(int kernel_id, float* total_ms, int* launches);
 int mi_transducer_profile_disable(void);
 

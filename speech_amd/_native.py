@@ -16,7 +16,7 @@ INCLUDE_DIR = os.path.join(os.path.dirname(_HERE), "include")
 LIB_PATH = os.environ.get("MI_TRANSDUCER_LIB") or os.path.join(CSRC_DIR, "libmi_transducer.so")
 SOURCES = [os.path.join(CSRC_DIR, "mi_transducer.hip")]
 
-ABI_VERSION = 2
+ABI_VERSION = 3
 SUCCESS, INVALID_VALUE, LAUNCH_FAILURE = 0, 1, 2
 DTYPE_F32, DTYPE_BF16, DTYPE_F16 = 0, 1, 2
 
@@ -70,7 +70,7 @@ _SIGNATURES = {
     "mi_transducer_export_lattice": [_vp, _c_size_t, _vp, _vp, _c_int, _c_int, _c_int, _c_int, _vp, _vp, _vp, _vp,
                                      _vp, _vp],
     "mi_transducer_length_maxima": [_vp, _vp, _c_int, _vp, _vp],
-    "mi_transducer_profile_enable": [_c_int],
+    "mi_transducer_profile_enable": [_c_int, ctypes.c_uint],
     "mi_transducer_profile_read": [_c_int, ctypes.POINTER(_c_float), ctypes.POINTER(_c_int)],
     "mi_transducer_profile_disable": [],
     "mi_transducer_copy_probe": [_vp, _vp, _c_size_t, _vp],
@@ -121,8 +121,12 @@ def workspace_bytes(B, T, U, D=0):
 PROFILE_KERNELS = {"denom_gather_kernel": 0, "lattice_kernel": 1, "cell_kernel": 2, "grad_stream_kernel": 3}
 
 
-def profile_enable(max_launches):
-    check_status(lib().mi_transducer_profile_enable(int(max_launches)), "profile_enable")
+def profile_enable(max_launches, kernels=None):
+    """Bracket the next launches of the named kernels (default: all) with HIP events."""
+    mask = 0
+    for name in kernels or PROFILE_KERNELS:
+        mask |= 1 << PROFILE_KERNELS[name]
+    check_status(lib().mi_transducer_profile_enable(int(max_launches), mask), "profile_enable")
 
 
 def profile_read():

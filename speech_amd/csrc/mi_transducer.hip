@@ -242,6 +242,19 @@ __device__ __forceinline__ unsigned logical_block() {
   return (turn / MI_XCD_SPAN) * (8u * MI_XCD_SPAN) + xcd * MI_XCD_SPAN + (turn % MI_XCD_SPAN);
 }
 
+#ifndef MI_NT_STORE
+#define MI_NT_STORE 0
+#endif
+__device__ __forceinline__ void store_stream(uint4* p, const uint4& v) {
+#if MI_NT_STORE
+  u32x4 x;
+  x.x = v.x; x.y = v.y; x.z = v.z; x.w = v.w;
+  __builtin_nontemporal_store(x, (u32x4*)p);
+#else
+  *p = v;
+#endif
+}
+
 // Which (b, t, u) row a wave works on.  Grid = (8 * ceil(U/4), ceil(B*T/8)): workgroups are
 // dealt round-robin to the 8 XCDs in linear-id order, so blockIdx.x & 7 names the XCD; each
 // XCD gets a contiguous eighth of the (b,t) rows and walks it in memory order.  Rows are not
@@ -1060,7 +1073,12 @@ __device__ __forceinline__ float wave_sum_u(float v) {
 #define MI_ROWS_PER_WAVE 1
 #endif
 constexpr int kRowsPerWave = MI_ROWS_PER_WAVE;
-constexpr int kChunkRows = kRowsPerBlock * kRowsPerWave;
+#ifndef MI_ROW_WAVES
+#define MI_ROW_WAVES 4
+#endif
+constexpr int kRowWaves = MI_ROW_WAVES;  // waves (= rows in flight) per workgroup of the row kernels
+constexpr int kRowThreads = 64 * kRowWaves;
+constexpr int kChunkRows = kRowWaves * kRowsPerWave;
 
 // zero-fills elements [e_begin, e_end) of `base` with the whole workgroup: 16-byte stores on
 // the aligned middle, element stores on the ragged ends
@@ -1079,11 +1097,11 @@ template <int DT> __device__ __forceinline__ void zero_elems(void* base, size_t 
   else if (tid >= 32 && tid - 32 < (int)(tail / BYTES)) Elem<DT>::store1(p1 - tail, tid - 32, 0.f);
   uint4* q = (uint4*)(p0 + head);
   const uint4 z = make_uint4(0, 0, 0, 0);
-  for (size_t i = tid; i < nvec; i += 256) q[i] = z;
+  for (size_t i = tid; i < nvec; i += kRowThreads) store_stream(q + i, z);
 }
 
 template <int DT, int R>
-__global__ __launch_bounds__(256) void denom_rows_kernel(
+__global__ __launch_bounds__(kRowThreads) void denom_rows_kernel(
     const void* __restrict__ acts, const int64_t* __restrict__ labels, const int64_t* __restrict__ act_lens,
     const int64_t* __restrict__ label_lens, float* __restrict__ denom, float* __restrict__ arcs, int T, int U, int V,
     int D, int blank, int ND, int Us, int A, int nchunks, int nblocks) {
@@ -1111,7 +1129,7 @@ __global__ __launch_bounds__(256) void denom_rows_kernel(
   int labs[kRowsPerWave];
 #pragma unroll
   for (int i = 0; i < kRowsPerWave; ++i) {
-    const int uu = u_begin + kRowsPerBlock * i;
+    const int uu = u_begin + kRowWaves * i;
     labs[i] = (uu < Ub - 1) ? clampi(labels[(size_t)b * (U - 1) + uu], 0, V - 1) : -1;
   }
 
@@ -1183,13 +1201,13 @@ __global__ __launch_bounds__(256) void denom_rows_kernel(
   fetch(u_begin, labs[0], cur);
 #pragma unroll
   for (int i = 0; i < kRowsPerWave; ++i) {
-    const int uu = u_begin + kRowsPerBlock * i;
+    const int uu = u_begin + kRowWaves * i;
     if (uu >= u_end) break;
     if (i + 1 < kRowsPerWave) {
       // always fetch (the last row of the wave re-reads itself): an unconditional load keeps the
       // wait counters exact, so reducing row i never waits for the loads of row i+1
-      const bool more = uu + kRowsPerBlock < u_end;
-      fetch(more ? uu + kRowsPerBlock : uu, more ? labs[i + 1] : labs[i], nxt);
+      const bool more = uu + kRowWaves < u_end;
+      fetch(more ? uu + kRowWaves : uu, more ? labs[i + 1] : labs[i], nxt);
     }
     reduce(uu, labs[i], cur);
     cur = nxt;
@@ -1199,7 +1217,7 @@ __global__ __launch_bounds__(256) void denom_rows_kernel(
 // FUSED (RNNT): the row's coefficients are derived here from the lattice state, one wave-uniform
 // evaluation per row, instead of being read from the coefficient buffer a cell kernel filled.
 template <int DT, int R, bool FUSED>
-__global__ __launch_bounds__(256) void grad_rows_kernel(const void* __restrict__ acts, void* __restrict__ grads,
+__global__ __launch_bounds__(kRowThreads) void grad_rows_kernel(const void* __restrict__ acts, void* __restrict__ grads,
                                                         const float* __restrict__ coef, LatticeView lv,
                                                         const int64_t* __restrict__ act_lens,
                                                         const int64_t* __restrict__ label_lens, int T, int U, int V,
@@ -1294,7 +1312,7 @@ __global__ __launch_bounds__(256) void grad_rows_kernel(const void* __restrict__
             if (first + i == lab) g[i] = gL;
           }
         }
-        gvp[64 * k] = Elem<DT>::pack(g);
+        store_stream(gvp + 64 * k, Elem<DT>::pack(g));
       }
     }
     const int v = extra_index(sp);
@@ -1314,9 +1332,9 @@ __global__ __launch_bounds__(256) void grad_rows_kernel(const void* __restrict__
   fetch(u_begin, cur);
 #pragma unroll
   for (int i = 0; i < kRowsPerWave; ++i) {
-    const int uu = u_begin + kRowsPerBlock * i;
+    const int uu = u_begin + kRowWaves * i;
     if (uu >= z0) break;
-    if (i + 1 < kRowsPerWave) fetch(uu + kRowsPerBlock < z0 ? uu + kRowsPerBlock : uu, nxt);
+    if (i + 1 < kRowsPerWave) fetch(uu + kRowWaves < z0 ? uu + kRowWaves : uu, nxt);
     emit(uu, cur);
     cur = nxt;
   }
@@ -1390,6 +1408,7 @@ __global__ __launch_bounds__(256) void length_maxima_kernel(const int64_t* __res
 struct ProfState {
   bool on = false;
   int cap = 0;
+  unsigned mask = ~0u;
   int count[MI_PROFILE_KERNELS] = {0, 0, 0, 0};
   std::vector<hipEvent_t> start[MI_PROFILE_KERNELS], stop[MI_PROFILE_KERNELS];
 };
@@ -1400,7 +1419,7 @@ struct ProfScope {
   hipStream_t stream;
   bool live;
   ProfScope(int kernel_id, hipStream_t s) : id(kernel_id), stream(s), live(false) {
-    if (g_prof.on && g_prof.count[id] < g_prof.cap) {
+    if (g_prof.on && ((g_prof.mask >> id) & 1u) && g_prof.count[id] < g_prof.cap) {
       live = true;
       (void)hipEventRecord(g_prof.start[id][g_prof.count[id]], stream);
     }
@@ -1516,7 +1535,7 @@ int run_denom(const Common& c) {
   const int R = rows_R(c);
   ProfScope prof(MI_PROFILE_DENOM, c.stream);
 #define LAUNCH_DENOM_ROWS(DT, RR)                                                                                   \
-  hipLaunchKernelGGL((denom_rows_kernel<DT, RR>), chunk_grid(c), dim3(256), 0, c.stream, c.acts, c.labels,           \
+  hipLaunchKernelGGL((denom_rows_kernel<DT, RR>), chunk_grid(c), dim3(kRowThreads), 0, c.stream, c.acts, c.labels,           \
                      c.act_lens, c.label_lens, denom, arcs, c.T, c.U, c.V, c.D, c.blank, L.ND, L.Us, L.A, chunks_of(c), chunk_blocks(c))
 #define LAUNCH_DENOM(DT)                                                                                            \
   do {                                                                                                              \
@@ -1624,11 +1643,11 @@ int run_grad_stream(const Common& c, void* grads, int zero_durations, bool fused
 #define LAUNCH_GRAD_ROWS(DT, RR)                                                                                    \
   do {                                                                                                              \
     if (fused)                                                                                                      \
-      hipLaunchKernelGGL((grad_rows_kernel<DT, RR, true>), chunk_grid(c), dim3(256), 0, c.stream, c.acts, grads,     \
+      hipLaunchKernelGGL((grad_rows_kernel<DT, RR, true>), chunk_grid(c), dim3(kRowThreads), 0, c.stream, c.acts, grads,     \
                          coef, lv, c.act_lens, c.label_lens, c.T, c.U, c.V, c.D, c.blank, L.CS, zero_durations,      \
                          chunks_of(c), chunk_blocks(c));                                                            \
     else                                                                                                            \
-      hipLaunchKernelGGL((grad_rows_kernel<DT, RR, false>), chunk_grid(c), dim3(256), 0, c.stream, c.acts, grads,    \
+      hipLaunchKernelGGL((grad_rows_kernel<DT, RR, false>), chunk_grid(c), dim3(kRowThreads), 0, c.stream, c.acts, grads,    \
                          coef, lv, c.act_lens, c.label_lens, c.T, c.U, c.V, c.D, c.blank, L.CS, zero_durations,      \
                          chunks_of(c), chunk_blocks(c));                                                            \
   } while (0)
@@ -1685,7 +1704,7 @@ int run_tdt_cells(const Common& c, const ScaleArg& sc, float lambda, float clamp
 // ----------------------------------------------------------------------------------------
 extern "C" {
 
-int mi_transducer_abi_version(void) { return 2; }
+int mi_transducer_abi_version(void) { return 3; }
 
 int mi_transducer_workspace_bytes(int B, int T, int U, int D, size_t* out_bytes) {
   Layout L;
@@ -1809,8 +1828,8 @@ int mi_transducer_length_maxima(const int64_t* act_lens, const int64_t* label_le
   return launch_status();
 }
 
-int mi_transducer_profile_enable(int max_launches) {
-  if (max_launches <= 0 || max_launches > 65536) return MI_TRANSDUCER_INVALID_VALUE;
+int mi_transducer_profile_enable(int max_launches, unsigned kernel_mask) {
+  if (max_launches <= 0 || max_launches > 65536 || kernel_mask == 0) return MI_TRANSDUCER_INVALID_VALUE;
   g_prof.on = false;
   for (int k = 0; k < MI_PROFILE_KERNELS; ++k) {
     while ((int)g_prof.start[k].size() < max_launches) {
@@ -1822,6 +1841,7 @@ int mi_transducer_profile_enable(int max_launches) {
     g_prof.count[k] = 0;
   }
   g_prof.cap = max_launches;
+  g_prof.mask = kernel_mask;
   g_prof.on = true;
   return MI_TRANSDUCER_SUCCESS;
 }
