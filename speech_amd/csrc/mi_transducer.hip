@@ -756,6 +756,180 @@ __global__ __launch_bounds__(64) void tdt_lattice_kernel(const float* __restrict
   }
 }
 
+// TDT lattice, workgroup version (gpu_rnnt_kernel.py:888-1241): one workgroup per (utterance,
+// direction), one thread per column u, one anti-diagonal per step, one barrier per step.
+//   alpha: a finished cell leaves its 2D outgoing arc scores (alpha + arc weight, blank arcs
+//          and label arcs per duration) in an LDS ring of R = max_duration + 2 diagonals; a
+//          cell's alpha is ONE log-sum-exp over the up to 2D-1 scores that land on it (max,
+//          sum of exp2 in fp32, one log), plus the reference's finite -10000 seeds.
+//   beta : the ring holds beta of the last R diagonals; arc weights are the cell's own.
+// The cell's arc weights (blank, label, D duration log-probs) do not depend on the recursion
+// and are fetched P diagonals ahead.
+template <int D>
+__global__ __launch_bounds__(256) void tdt_lattice_block_kernel(
+    const float* __restrict__ arcs, double* __restrict__ alphas, double* __restrict__ betas, double* __restrict__ ll,
+    float* __restrict__ costs, const int64_t* __restrict__ act_lens, const int64_t* __restrict__ label_lens, int T,
+    int U, int ND, int Us, float cost_scale, int with_betas, TdtParams prm) {
+  constexpr int A = 2 + D;
+  constexpr int P = 4;
+  extern __shared__ double ring[];
+  const int b = with_betas ? (int)(blockIdx.x >> 1) : (int)blockIdx.x;
+  const int dir = with_betas ? (int)(blockIdx.x & 1) : 0;
+  const int u = threadIdx.x;  // blockDim.x == Us
+  const int Tb = clampi(act_lens[b], 1, T);
+  const int Ub = clampi(label_lens[b] + 1, 1, U);
+  const int nd = Tb + Ub - 1;
+  const int R = prm.R;
+  const double sigma = (double)prm.sigma;
+  const double NEG = kTdtNeg;
+  int dur[D];
+#pragma unroll
+  for (int i = 0; i < D; ++i) dur[i] = prm.dur[i];
+  const size_t row_pitch = (size_t)A * Us;
+  const float* arcs_b = arcs + (size_t)b * ND * row_pitch + u;
+
+  auto load_rows = [&](int nfirst, int step, float(&W)[P][A]) {
+#pragma unroll
+    for (int p = 0; p < P; ++p) {
+      int n = nfirst + step * p;
+      n = n < 0 ? 0 : (n >= nd ? nd - 1 : n);
+      const float* rp = arcs_b + (size_t)n * row_pitch;
+#pragma unroll
+      for (int a = 0; a < A; ++a) W[p][a] = rp[(size_t)a * Us];
+    }
+  };
+  // log-sum-exp of x[0..N) (entries may be -inf = absent) and `seeds` copies of the sentinel
+  auto lse_all = [&](const double* x, int seeds) {
+    double m = seeds > 0 ? NEG : -INFINITY;
+#pragma unroll
+    for (int i = 0; i < 2 * D; ++i) m = fmax(m, x[i]);
+    float s = (float)seeds * fast_exp2((float)(NEG - m) * kLog2e);
+#pragma unroll
+    for (int i = 0; i < 2 * D; ++i) s += fast_exp2((float)(x[i] - m) * kLog2e);
+    return m + (double)(__builtin_amdgcn_logf(s) * 0.6931471805599453f);
+  };
+
+  if (dir == 0) {
+    for (int i = u; i < R * 2 * D * Us; i += Us) ring[i] = NEG;
+    __syncthreads();
+    double* out = alphas + (size_t)b * ND * Us + u;
+    double ll_acc = NEG;
+    int cur = 0;  // n % R, kept incrementally (R is a run-time value: no divisions in the loop)
+    auto step_fn = [&](int n, const float* w) {
+      const int t = n - u;
+      double x[2 * D];
+#pragma unroll
+      for (int i = 0; i < D; ++i) {
+        const int d = dur[i];
+        int sb = cur - d, sl = cur - 1 - d;  // slots of diagonals n-d and n-1-d
+        sb += sb < 0 ? R : 0;
+        sl += sl < 0 ? R : 0;
+        const double vb = ring[((sb * 2 * D) + i) * Us + u];
+        const double vl = ring[((sl * 2 * D) + D + i) * Us + (u > 0 ? u - 1 : 0)];
+        x[i] = (d > 0 && t >= d) ? vb : -INFINITY;
+        x[D + i] = (u > 0 && t >= d) ? vl : -INFINITY;
+      }
+      double a;
+      if (t == 0 && u == 0) a = 0.0;
+      else if (t == 0) a = (dur[0] == 0) ? x[D] : NEG;  // only a duration-0 label arc reaches row 0 (:941-955)
+      else a = lse_all(x, u == 0 ? 1 : 2);              // the emit and the no-emit accumulator are both seeded
+      out[(size_t)n * Us] = a;
+      const double wb = a + (double)w[0], wl = a + (double)w[1];
+      double* slot = ring + (size_t)(cur * 2 * D) * Us + u;
+#pragma unroll
+      for (int i = 0; i < D; ++i) {
+        const double dl = (double)w[2 + i];
+        const double ob = (wb - sigma) + dl;
+        slot[(size_t)i * Us] = ob;
+        slot[(size_t)(D + i) * Us] = (wl - sigma) + dl;
+        if (dur[i] > 0 && u == Ub - 1 && t >= 0 && t + dur[i] == Tb) ll_acc = lse_h(ll_acc, ob);  // :1040-1071
+      }
+      cur = cur + 1 == R ? 0 : cur + 1;
+      __syncthreads();
+    };
+    float wa[P][A], wb[P][A];
+    int n0 = 0;
+    load_rows(0, 1, wa);
+    for (; n0 + 2 * P <= nd; n0 += 2 * P) {
+      load_rows(n0 + P, 1, wb);
+#pragma unroll
+      for (int p = 0; p < P; ++p) step_fn(n0 + p, wa[p]);
+      load_rows(n0 + 2 * P, 1, wa);
+#pragma unroll
+      for (int p = 0; p < P; ++p) step_fn(n0 + P + p, wb[p]);
+    }
+    for (; n0 < nd; ++n0) {
+      float w[A];
+#pragma unroll
+      for (int a = 0; a < A; ++a) w[a] = arcs_b[(size_t)n0 * row_pitch + (size_t)a * Us];
+      step_fn(n0, w);
+    }
+    if (u == Ub - 1) {
+      ll[2 * b] = ll_acc;
+      costs[b] = -(float)ll_acc * cost_scale;
+    }
+  } else {
+    for (int i = u; i < R * Us; i += Us) ring[i] = NEG;
+    __syncthreads();
+    double* out = betas + (size_t)b * ND * Us + u;
+    double last = NEG;
+    int cur = (nd - 1) % R;  // n % R, kept incrementally
+    auto step_fn = [&](int n, const float* w) {
+      const int t = n - u;
+      const double lpb = (double)w[0], lpl = (double)w[1];
+      double x[2 * D];
+#pragma unroll
+      for (int i = 0; i < D; ++i) {
+        const int d = dur[i];
+        const double dl = (double)w[2 + i];
+        const double bw = (lpb + dl) - sigma, lw = (lpl + dl) - sigma;
+        int sb = cur + d, sl = cur + d + 1;  // slots of diagonals n+d and n+d+1
+        sb -= sb >= R ? R : 0;
+        sl -= sl >= R ? R : 0;
+        const double vb = ring[sb * Us + u];
+        const double vl = ring[sl * Us + (u + 1 < Us ? u + 1 : u)];
+        double xb = -INFINITY;
+        if (d > 0) {
+          if (t + d < Tb) xb = vb + bw;
+          else if (t + d == Tb && u == Ub - 1) xb = bw;
+        }
+        x[i] = xb;
+        x[D + i] = (t + d < Tb && u + 1 < Ub) ? vl + lw : -INFINITY;
+      }
+      double v;
+      double corner = NEG;  // the corner ends the utterance with one blank of duration 1 (:1137-1148)
+#pragma unroll
+      for (int i = 0; i < D; ++i) corner = (i == prm.one_idx) ? x[i] : corner;
+      if (t == Tb - 1 && u == Ub - 1) v = corner;
+      else if (t == Tb - 1 && u < Ub - 1) v = (dur[0] == 0) ? x[D] : NEG;  // last row: duration-0 labels only
+      else v = lse_all(x, u == Ub - 1 ? 1 : 2);
+      out[(size_t)n * Us] = v;
+      ring[cur * Us + u] = v;
+      last = v;
+      cur = cur == 0 ? R - 1 : cur - 1;
+      __syncthreads();
+    };
+    float wa[P][A], wb[P][A];
+    int n0 = nd - 1;
+    load_rows(n0, -1, wa);
+    for (; n0 - 2 * P + 1 >= 0; n0 -= 2 * P) {
+      load_rows(n0 - P, -1, wb);
+#pragma unroll
+      for (int p = 0; p < P; ++p) step_fn(n0 - p, wa[p]);
+      load_rows(n0 - 2 * P, -1, wa);
+#pragma unroll
+      for (int p = 0; p < P; ++p) step_fn(n0 - P - p, wb[p]);
+    }
+    for (; n0 >= 0; --n0) {
+      float w[A];
+#pragma unroll
+      for (int a = 0; a < A; ++a) w[a] = arcs_b[(size_t)n0 * row_pitch + (size_t)a * Us];
+      step_fn(n0, w);
+    }
+    if (u == 0) ll[2 * b + 1] = last;  // beta(0,0)
+  }
+}
+
 // ----------------------------------------------------------------------------------------
 // Per-cell gradient coefficients.  For a valid cell the gradient row is
 //   g_v = clamp( p_v * W  - [v = blank] PB - [v = label] PL ) * scale,   p_v = exp(x_v + denom)
@@ -1590,18 +1764,37 @@ int run_tdt_lattice(const Common& c, float* costs, float lambda, int with_betas,
   double* betas = (double*)(c.ws + L.off_betas);
   double* ll = (double*)(c.ws + L.off_ll);
   const unsigned grid = (unsigned)(with_betas ? 2 * c.B : c.B);
-  const size_t lds = (size_t)2 * prm.R * L.Us * sizeof(double);
-  if (lds > 160 * 1024) return MI_TRANSDUCER_INVALID_VALUE;
   ProfScope prof(MI_PROFILE_LATTICE, c.stream);
+  // workgroup version: one thread per column, all of a cell's arcs in one log-sum-exp
+  const size_t lds_block = (size_t)prm.R * 2 * prm.D * L.Us * sizeof(double);
+  if (prm.D <= 8 && L.Us <= 256 && lds_block <= 160 * 1024) {
+#define LAUNCH_TBLK(DD)                                                                                              \
+  if (lds_block > 48 * 1024 &&                                                                                       \
+      hipFuncSetAttribute((const void*)tdt_lattice_block_kernel<DD>, hipFuncAttributeMaxDynamicSharedMemorySize,     \
+                          (int)lds_block) != hipSuccess)                                                             \
+    return MI_TRANSDUCER_LAUNCH_FAILURE;                                                                             \
+  hipLaunchKernelGGL(tdt_lattice_block_kernel<DD>, dim3(grid), dim3(L.Us), lds_block, c.stream, arcs, alphas, betas,  \
+                     ll, costs, c.act_lens, c.label_lens, c.T, c.U, L.ND, L.Us, cost_scale_of(lambda), with_betas,   \
+                     prm)
+    switch (prm.D) {
+      case 1: LAUNCH_TBLK(1); break;
+      case 2: LAUNCH_TBLK(2); break;
+      case 3: LAUNCH_TBLK(3); break;
+      case 4: LAUNCH_TBLK(4); break;
+      case 5: LAUNCH_TBLK(5); break;
+      case 6: LAUNCH_TBLK(6); break;
+      case 7: LAUNCH_TBLK(7); break;
+      default: LAUNCH_TBLK(8); break;
+    }
+#undef LAUNCH_TBLK
+    return launch_status();
+  }
+  // general fallback (many durations or a very wide label axis): one wave per lattice
+  const size_t lds = (size_t)2 * prm.R * L.Us * sizeof(double);
+  if (lds > 64 * 1024) return MI_TRANSDUCER_INVALID_VALUE;
 #define LAUNCH_TLAT(KK)                                                                                              \
-  do {                                                                                                               \
-    if (lds > 48 * 1024 &&                                                                                           \
-        hipFuncSetAttribute((const void*)tdt_lattice_kernel<KK>, hipFuncAttributeMaxDynamicSharedMemorySize,         \
-                            (int)lds) != hipSuccess)                                                                 \
-      return MI_TRANSDUCER_LAUNCH_FAILURE;                                                                           \
-    hipLaunchKernelGGL(tdt_lattice_kernel<KK>, dim3(grid), dim3(64), lds, c.stream, arcs, alphas, betas, ll, costs,  \
-                       c.act_lens, c.label_lens, c.T, c.U, L.ND, L.A, cost_scale_of(lambda), with_betas, prm);       \
-  } while (0)
+  hipLaunchKernelGGL(tdt_lattice_kernel<KK>, dim3(grid), dim3(64), lds, c.stream, arcs, alphas, betas, ll, costs,    \
+                     c.act_lens, c.label_lens, c.T, c.U, L.ND, L.A, cost_scale_of(lambda), with_betas, prm)
   switch (L.K) {
     case 1: LAUNCH_TLAT(1); break;
     case 2: LAUNCH_TLAT(2); break;
