@@ -31,7 +31,10 @@ HBM_PEAK_GBPS = 8000.0  # MI355X HBM3E, published peak
 # HBM bytes per launch of grad_stream_kernel from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of
 # this script, scaled by what the same counters read for mi_transducer_copy_probe of known size
 # (summaries under profiles/).  None = not measured for that workload.
-MEASURED_TRAFFIC_BYTES = {}
+MEASURED_TRAFFIC_BYTES = {
+    # profiles/transducer_kernels_cfg2_hbm_traffic.md: fetch 1.6316 GB + write 2.9804 GB
+    "cfg2_rnnt_B16_T375_U121_V1025_f32": 4612065338,
+}
 
 
 def parse_args():
@@ -41,7 +44,7 @@ def parse_args():
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--workload", type=int, default=1, help="index into speech_amd.synthetic.CONFIGS (1 = north star)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
-    ap.add_argument("--cpu-sample-utterances", type=int, default=8)
+    ap.add_argument("--cpu-sample-utterances", type=int, default=16)
     return ap.parse_args()
 
 
