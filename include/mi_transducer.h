@@ -74,11 +74,13 @@ int mi_rnnt_forward(const void* acts, int act_dtype, const int64_t* labels, cons
  * which folds the autograd backward `grads.mul_(grad_output)` (rnnt_pytorch.py:88-92; a
  * broadcast grad_output is stride 0) and the 'mean' reduction's 1/B (rnnt_pytorch.py:77-81)
  * into the same pass.  grad_scale: device float32, nullable; grad_scale_stride >= 0 in elements.
- * Must follow mi_rnnt_forward(with_betas != 0) on the same workspace and inputs. */
+ * Must follow mi_rnnt_forward(with_betas != 0) on the same workspace and inputs.
+ * padding_zeroed != 0: the padded cells of grads were already zero-filled by
+ * mi_transducer_zero_padding (the caller made this call wait for it); they are then skipped. */
 int mi_rnnt_backward(const void* acts, int act_dtype, const int64_t* labels, const int64_t* act_lens,
                      const int64_t* label_lens, void* grads, const float* grad_scale, int grad_scale_stride,
-                     float grad_mul, int B, int T, int U, int V, int blank, float fastemit_lambda, float clamp,
-                     void* workspace, size_t workspace_bytes, void* stream);
+                     float grad_mul, int padding_zeroed, int B, int T, int U, int V, int blank,
+                     float fastemit_lambda, float clamp, void* workspace, size_t workspace_bytes, void* stream);
 
 /* rnnt_loss_gpu in one call (rnnt.py:138-236 -> GPURNNT.cost_and_grad / score_forward,
  * gpu_rnnt.py:125-265): grads == NULL means forward only. */
@@ -105,15 +107,40 @@ int mi_tdt_forward(const void* acts, int act_dtype, const int64_t* labels, const
 
 int mi_tdt_backward(const void* acts, int act_dtype, const int64_t* labels, const int64_t* act_lens,
                     const int64_t* label_lens, void* grads, const float* grad_scale, int grad_scale_stride,
-                    float grad_mul, int B, int T, int U, int V, int D, const int32_t* durations_host, int blank,
-                    float fastemit_lambda, float clamp, float sigma, int use_plain_rnnt, void* workspace,
-                    size_t workspace_bytes, void* stream);
+                    float grad_mul, int padding_zeroed, int B, int T, int U, int V, int D,
+                    const int32_t* durations_host, int blank, float fastemit_lambda, float clamp, float sigma,
+                    int use_plain_rnnt, void* workspace, size_t workspace_bytes, void* stream);
 
 int mi_tdt_loss(const void* acts, int act_dtype, const int64_t* labels, const int64_t* act_lens,
                 const int64_t* label_lens, float* costs, void* grads, const float* grad_scale, int grad_scale_stride,
                 float grad_mul, int B, int T, int U, int V, int D, const int32_t* durations_host, int blank,
                 float fastemit_lambda, float clamp, float sigma, int use_plain_rnnt, void* workspace,
                 size_t workspace_bytes, void* stream);
+
+/* The two stages of a forward call on their own (mi_rnnt_forward = denominators + rnnt lattice,
+ * mi_tdt_forward = denominators + tdt lattice), for callers that want to order other work between
+ * them and for stage-level tests.  They mirror the reference's separately launched kernels:
+ * reduce_max/reduce_exp (utils/cuda_utils/reduce.py:299-362) and compute_alphas/betas_kernel
+ * (utils/cuda_utils/gpu_rnnt_kernel.py:73-269, :888-1241).  D = 0 for RNNT; the lattice calls need
+ * the D the denominators were run with (it fixes the workspace layout). */
+int mi_transducer_denominators(const void* acts, int act_dtype, const int64_t* labels, const int64_t* act_lens,
+                               const int64_t* label_lens, int B, int T, int U, int V, int D, int blank,
+                               void* workspace, size_t workspace_bytes, void* stream);
+int mi_rnnt_lattice(const int64_t* act_lens, const int64_t* label_lens, float* costs, int B, int T, int U, int D,
+                    float fastemit_lambda, int with_betas, void* workspace, size_t workspace_bytes, void* stream);
+int mi_tdt_lattice(const int64_t* act_lens, const int64_t* label_lens, float* costs, int B, int T, int U, int D,
+                   const int32_t* durations_host, float fastemit_lambda, float sigma, int with_betas, void* workspace,
+                   size_t workspace_bytes, void* stream);
+
+/* Zero-fills the gradient entries of every padded cell (t >= act_lens[b] or u > label_lens[b]) of
+ * grads[B,T,U,VD] and touches nothing else.  The reference zero-fills the whole gradient tensor up
+ * front (zeros_like, rnnt_pytorch.py:58; `grads *= 0`, gpu_rnnt.py:156); this is the part of that
+ * work which survives, split out because it depends on the lengths only: enqueued on a second
+ * stream after the denominators it fills the time HBM idles during the lattice recursion; the
+ * backward call is then told padding_zeroed = 1 and may even run beside it (the two write disjoint
+ * bytes).  Ordering between the streams, and the final join, are the caller's job. */
+int mi_transducer_zero_padding(void* grads, int act_dtype, const int64_t* act_lens, const int64_t* label_lens, int B,
+                               int T, int U, int VD, void* stream);
 
 /* Stage-level read-out for kernel parity tests (the reference tests launch each
  * kernel on its own, tests/collections/asr/numba/rnnt_loss/utils/test_gpu_rnnt_kernel.py):
@@ -140,11 +167,12 @@ int mi_transducer_length_maxima(const int64_t* act_lens, const int64_t* label_le
  * select only the kernel it needs.  mi_transducer_profile_read waits for the recorded
  * launches of one kernel class, returns their summed duration and count, and resets that
  * class.  Not thread-safe; leave disabled outside benchmarks. */
-#define MI_PROFILE_DENOM 0   /* denom_gather_kernel */
+#define MI_PROFILE_DENOM 0   /* denom_rows_kernel / denom_gather_kernel */
 #define MI_PROFILE_LATTICE 1 /* rnnt_lattice_kernel / tdt_lattice_kernel */
 #define MI_PROFILE_CELL 2    /* rnnt_cell_kernel / tdt_cell_kernel */
-#define MI_PROFILE_GRAD 3    /* grad_stream_kernel */
-#define MI_PROFILE_KERNELS 4
+#define MI_PROFILE_GRAD 3    /* grad_rows_kernel / grad_stream_kernel */
+#define MI_PROFILE_ZERO 4    /* zero_padding_kernel */
+#define MI_PROFILE_KERNELS 5
 int mi_transducer_profile_enable(int max_launches, unsigned kernel_mask);
 int mi_transducer_profile_read(int kernel_id, float* total_ms, int* launches);
 int mi_transducer_profile_disable(void);

@@ -16,7 +16,7 @@ INCLUDE_DIR = os.path.join(os.path.dirname(_HERE), "include")
 LIB_PATH = os.environ.get("MI_TRANSDUCER_LIB") or os.path.join(CSRC_DIR, "libmi_transducer.so")
 SOURCES = [os.path.join(CSRC_DIR, "mi_transducer.hip")]
 
-ABI_VERSION = 3
+ABI_VERSION = 5
 SUCCESS, INVALID_VALUE, LAUNCH_FAILURE = 0, 1, 2
 DTYPE_F32, DTYPE_BF16, DTYPE_F16 = 0, 1, 2
 
@@ -58,18 +58,24 @@ _SIGNATURES = {
     "mi_rnnt_forward": [_vp, _c_int, _vp, _vp, _vp, _vp, _c_int, _c_int, _c_int, _c_int, _c_int, _c_float, _c_int,
                         _vp, _c_size_t, _vp],
     "mi_rnnt_backward": [_vp, _c_int, _vp, _vp, _vp, _vp, _vp, _c_int, _c_float, _c_int, _c_int, _c_int, _c_int,
-                         _c_int, _c_float, _c_float, _vp, _c_size_t, _vp],
+                         _c_int, _c_int, _c_float, _c_float, _vp, _c_size_t, _vp],
     "mi_rnnt_loss": [_vp, _c_int, _vp, _vp, _vp, _vp, _vp, _vp, _c_int, _c_float, _c_int, _c_int, _c_int, _c_int,
                      _c_int, _c_float, _c_float, _vp, _c_size_t, _vp],
     "mi_tdt_forward": [_vp, _c_int, _vp, _vp, _vp, _vp, _c_int, _c_int, _c_int, _c_int, _c_int, _vp, _c_int, _c_float,
                        _c_float, _c_int, _c_int, _vp, _c_size_t, _vp],
     "mi_tdt_backward": [_vp, _c_int, _vp, _vp, _vp, _vp, _vp, _c_int, _c_float, _c_int, _c_int, _c_int, _c_int,
-                        _c_int, _vp, _c_int, _c_float, _c_float, _c_float, _c_int, _vp, _c_size_t, _vp],
+                        _c_int, _c_int, _vp, _c_int, _c_float, _c_float, _c_float, _c_int, _vp, _c_size_t, _vp],
     "mi_tdt_loss": [_vp, _c_int, _vp, _vp, _vp, _vp, _vp, _vp, _c_int, _c_float, _c_int, _c_int, _c_int, _c_int,
                     _c_int, _vp, _c_int, _c_float, _c_float, _c_float, _c_int, _vp, _c_size_t, _vp],
     "mi_transducer_export_lattice": [_vp, _c_size_t, _vp, _vp, _c_int, _c_int, _c_int, _c_int, _vp, _vp, _vp, _vp,
                                      _vp, _vp],
     "mi_transducer_length_maxima": [_vp, _vp, _c_int, _vp, _vp],
+    "mi_transducer_denominators": [_vp, _c_int, _vp, _vp, _vp, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _vp,
+                                   _c_size_t, _vp],
+    "mi_rnnt_lattice": [_vp, _vp, _vp, _c_int, _c_int, _c_int, _c_int, _c_float, _c_int, _vp, _c_size_t, _vp],
+    "mi_tdt_lattice": [_vp, _vp, _vp, _c_int, _c_int, _c_int, _c_int, _vp, _c_float, _c_float, _c_int, _vp, _c_size_t,
+                       _vp],
+    "mi_transducer_zero_padding": [_vp, _c_int, _vp, _vp, _c_int, _c_int, _c_int, _c_int, _vp],
     "mi_transducer_profile_enable": [_c_int, ctypes.c_uint],
     "mi_transducer_profile_read": [_c_int, ctypes.POINTER(_c_float), ctypes.POINTER(_c_int)],
     "mi_transducer_profile_disable": [],
@@ -118,7 +124,13 @@ def workspace_bytes(B, T, U, D=0):
     return int(out.value)
 
 
-PROFILE_KERNELS = {"denom_gather_kernel": 0, "lattice_kernel": 1, "cell_kernel": 2, "grad_stream_kernel": 3}
+PROFILE_KERNELS = {
+    "denom_gather_kernel": 0,
+    "lattice_kernel": 1,
+    "cell_kernel": 2,
+    "grad_stream_kernel": 3,
+    "zero_padding_kernel": 4,
+}
 
 
 def profile_enable(max_launches, kernels=None):

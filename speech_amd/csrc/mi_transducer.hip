@@ -49,7 +49,11 @@ constexpr float kLog2e = 1.4426950408889634f;
 constexpr float kNegInf = -INFINITY;
 constexpr double kTdtNeg = -10000.0;  // gpu_rnnt_kernel.py:38
 constexpr int kRowsPerBlock = 4;      // one wave per row, 256-thread blocks
-constexpr int kCoefBase = 8;          // floats per cell before the duration-gradient block
+constexpr int kCoefBase = 8;
+// flags of the gradient pass
+constexpr int kFlagZeroDurations = 1;  // omega branch of TDT: the duration block of the gradient is zero
+constexpr int kFlagPaddingDone = 2;    // padded cells were already zero-filled (mi_transducer_zero_padding)
+          // floats per cell before the duration-gradient block
 
 // ----------------------------------------------------------------------------------------
 // Workspace layout
@@ -1099,14 +1103,14 @@ __global__ __launch_bounds__(256) void tdt_cell_kernel(
 // ----------------------------------------------------------------------------------------
 // Pass 2: the gradient stream.  Grid (ceil(U/4), T, B), one wave per row; reads the V token
 // logits of valid rows, writes V + D gradient elements of every row.  Same kernel for RNNT
-// (D = 0) and TDT.  zero_durations: the omega branch of TDT -- duration gradients are zero.
+// (D = 0) and TDT.  flags: kFlagZeroDurations, kFlagPaddingDone.
 // ----------------------------------------------------------------------------------------
 template <int DT>
 __global__ __launch_bounds__(256) void grad_stream_kernel(const void* __restrict__ acts, void* __restrict__ grads,
                                                           const float* __restrict__ coef,
                                                           const int64_t* __restrict__ act_lens,
                                                           const int64_t* __restrict__ label_lens, int T, int U, int V,
-                                                          int D, int blank, int CS, int zero_durations, int BT,
+                                                          int D, int blank, int CS, int flags, int BT,
                                                           int bt_chunk) {
   constexpr int VEC = Elem<DT>::VEC;
   constexpr int R = 4;
@@ -1128,6 +1132,7 @@ __global__ __launch_bounds__(256) void grad_stream_kernel(const void* __restrict
   const bool same_phase = (int)((g0 & 15) / Elem<DT>::BYTES) == win.mis;
 
   if (t >= Tb || u >= Ub) {  // padded cell: zeros over all V + D entries
+    if (flags & kFlagPaddingDone) return;
     const RowSplit<DT> sp(win.mis, VD);
     const uint4 z = make_uint4(0, 0, 0, 0);
     if (same_phase) {
@@ -1165,7 +1170,7 @@ __global__ __launch_bounds__(256) void grad_stream_kernel(const void* __restrict
     if (v >= 0) {
       float g;
       if (v < V) g = token_grad(Elem<DT>::load1(acts, e0 + v), v);
-      else g = zero_durations ? 0.f : c[kCoefBase + v - V];
+      else g = (flags & kFlagZeroDurations) ? 0.f : c[kCoefBase + v - V];
       Elem<DT>::store1(grads, e0 + v, g);
     }
   }
@@ -1395,7 +1400,7 @@ __global__ __launch_bounds__(kRowThreads) void grad_rows_kernel(const void* __re
                                                         const float* __restrict__ coef, LatticeView lv,
                                                         const int64_t* __restrict__ act_lens,
                                                         const int64_t* __restrict__ label_lens, int T, int U, int V,
-                                                        int D, int blank, int CS, int zero_durations, int nchunks,
+                                                        int D, int blank, int CS, int flags, int nchunks,
                                                         int nblocks) {
   constexpr int VEC = Elem<DT>::VEC;
   const int lane = threadIdx.x & 63;
@@ -1416,7 +1421,7 @@ __global__ __launch_bounds__(kRowThreads) void grad_rows_kernel(const void* __re
   const int c1 = min(U, c0 + kChunkRows);
   // rows [c0, z0) of this chunk carry a gradient, rows [z0, c1) are padding: one contiguous range of zeros
   const int z0 = (t >= Tb) ? c0 : max(c0, min(Ub, c1));
-  zero_elems<DT>(grads, (cell0 + z0) * VD, (cell0 + c1) * VD);
+  if (!(flags & kFlagPaddingDone)) zero_elems<DT>(grads, (cell0 + z0) * VD, (cell0 + c1) * VD);
   const int u_begin = c0 + wave;
   if (u_begin >= z0) return;
   float scale = 1.f;
@@ -1491,7 +1496,7 @@ __global__ __launch_bounds__(kRowThreads) void grad_rows_kernel(const void* __re
     }
     const int v = extra_index(sp);
     if (v >= 0) {
-      float g = zero_durations ? 0.f : d.gd;
+      float g = (flags & kFlagZeroDurations) ? 0.f : d.gd;
       if (v < V) {
         g = stream_exp2(fmaf(d.xe, kLog2e, dl2)) * W;
         if (clamp_on) g = clamp_sym(g, cb);
@@ -1512,6 +1517,27 @@ __global__ __launch_bounds__(kRowThreads) void grad_rows_kernel(const void* __re
     emit(uu, cur);
     cur = nxt;
   }
+}
+
+// Zero-fill of the padded cells only (every row with t >= T_b or u >= U_b): a function of the
+// lengths alone, so it can run on another stream while the lattice recursion runs and HBM
+// would otherwise idle.  Same chunk order as the gradient pass.
+template <int DT>
+__global__ __launch_bounds__(kRowThreads) void zero_padding_kernel(void* __restrict__ grads,
+                                                                   const int64_t* __restrict__ act_lens,
+                                                                   const int64_t* __restrict__ label_lens, int T,
+                                                                   int U, int VD, int nchunks, int nblocks) {
+  const unsigned wg = logical_block();
+  if (wg >= (unsigned)nblocks) return;
+  const unsigned bt = wg / (unsigned)nchunks, chunk = wg - bt * (unsigned)nchunks;
+  const int b = (int)(bt / (unsigned)T), t = (int)(bt - (unsigned)b * (unsigned)T);
+  const int Tb = clampi(act_lens[b], 1, T);
+  const int Ub = clampi(label_lens[b] + 1, 1, U);
+  const size_t cell0 = ((size_t)b * T + t) * U;
+  const int c0 = (int)chunk * kChunkRows;
+  const int c1 = min(U, c0 + kChunkRows);
+  const int z0 = (t >= Tb) ? c0 : max(c0, min(Ub, c1));
+  zero_elems<DT>(grads, (cell0 + z0) * VD, (cell0 + c1) * VD);
 }
 
 // ----------------------------------------------------------------------------------------
@@ -1583,7 +1609,7 @@ struct ProfState {
   bool on = false;
   int cap = 0;
   unsigned mask = ~0u;
-  int count[MI_PROFILE_KERNELS] = {0, 0, 0, 0};
+  int count[MI_PROFILE_KERNELS] = {};
   std::vector<hipEvent_t> start[MI_PROFILE_KERNELS], stop[MI_PROFILE_KERNELS];
 };
 ProfState g_prof;
@@ -1814,7 +1840,7 @@ struct ScaleArg {
 
 // fused != 0: RNNT rows derive their coefficients from the lattice state inside the pass
 // (needs no cell kernel); only the register-resident row kernels can do that
-int run_grad_stream(const Common& c, void* grads, int zero_durations, bool fused, const ScaleArg& sc, float lambda,
+int run_grad_stream(const Common& c, void* grads, int flags, bool fused, const ScaleArg& sc, float lambda,
                     float clamp) {
   const Layout& L = c.L;
   const float* coef = (const float*)(c.ws + L.off_coef);
@@ -1837,11 +1863,11 @@ int run_grad_stream(const Common& c, void* grads, int zero_durations, bool fused
   do {                                                                                                              \
     if (fused)                                                                                                      \
       hipLaunchKernelGGL((grad_rows_kernel<DT, RR, true>), chunk_grid(c), dim3(kRowThreads), 0, c.stream, c.acts, grads,     \
-                         coef, lv, c.act_lens, c.label_lens, c.T, c.U, c.V, c.D, c.blank, L.CS, zero_durations,      \
+                         coef, lv, c.act_lens, c.label_lens, c.T, c.U, c.V, c.D, c.blank, L.CS, flags,               \
                          chunks_of(c), chunk_blocks(c));                                                            \
     else                                                                                                            \
       hipLaunchKernelGGL((grad_rows_kernel<DT, RR, false>), chunk_grid(c), dim3(kRowThreads), 0, c.stream, c.acts, grads,    \
-                         coef, lv, c.act_lens, c.label_lens, c.T, c.U, c.V, c.D, c.blank, L.CS, zero_durations,      \
+                         coef, lv, c.act_lens, c.label_lens, c.T, c.U, c.V, c.D, c.blank, L.CS, flags,               \
                          chunks_of(c), chunk_blocks(c));                                                            \
   } while (0)
 #define LAUNCH_GRAD(DT)                                                                                             \
@@ -1853,7 +1879,7 @@ int run_grad_stream(const Common& c, void* grads, int zero_durations, bool fused
       case 8: LAUNCH_GRAD_ROWS(DT, 8); break;                                                                       \
       default:                                                                                                      \
         hipLaunchKernelGGL(grad_stream_kernel<DT>, g.grid, dim3(256), 0, c.stream, c.acts, grads, coef, c.act_lens, \
-                           c.label_lens, c.T, c.U, c.V, c.D, c.blank, L.CS, zero_durations, g.BT, g.bt_chunk);      \
+                           c.label_lens, c.T, c.U, c.V, c.D, c.blank, L.CS, flags, g.BT, g.bt_chunk);               \
     }                                                                                                               \
   } while (0)
   if (c.dt == MI_DTYPE_F32) LAUNCH_GRAD(MI_DTYPE_F32);
@@ -1897,7 +1923,7 @@ int run_tdt_cells(const Common& c, const ScaleArg& sc, float lambda, float clamp
 // ----------------------------------------------------------------------------------------
 extern "C" {
 
-int mi_transducer_abi_version(void) { return 3; }
+int mi_transducer_abi_version(void) { return 5; }
 
 int mi_transducer_workspace_bytes(int B, int T, int U, int D, size_t* out_bytes) {
   Layout L;
@@ -1920,8 +1946,8 @@ int mi_rnnt_forward(const void* acts, int act_dtype, const int64_t* labels, cons
 
 int mi_rnnt_backward(const void* acts, int act_dtype, const int64_t* labels, const int64_t* act_lens,
                      const int64_t* label_lens, void* grads, const float* grad_scale, int grad_scale_stride,
-                     float grad_mul, int B, int T, int U, int V, int blank, float fastemit_lambda, float clamp,
-                     void* workspace, size_t workspace_bytes, void* stream) {
+                     float grad_mul, int padding_zeroed, int B, int T, int U, int V, int blank,
+                     float fastemit_lambda, float clamp, void* workspace, size_t workspace_bytes, void* stream) {
   Common c;
   if (!grads || clamp < 0.f || grad_scale_stride < 0) return MI_TRANSDUCER_INVALID_VALUE;
   int st = check_common(acts, act_dtype, labels, act_lens, label_lens, B, T, U, V, 0, blank, workspace,
@@ -1930,7 +1956,7 @@ int mi_rnnt_backward(const void* acts, int act_dtype, const int64_t* labels, con
   const ScaleArg sc = {grad_scale, grad_scale_stride, grad_mul};
   const bool fused = grad_rows_R(c, grads) != 0;
   if (!fused && (st = run_rnnt_cells(c, sc, fastemit_lambda, clamp))) return st;
-  return run_grad_stream(c, grads, 0, fused, sc, fastemit_lambda, clamp);
+  return run_grad_stream(c, grads, padding_zeroed ? kFlagPaddingDone : 0, fused, sc, fastemit_lambda, clamp);
 }
 
 int mi_rnnt_loss(const void* acts, int act_dtype, const int64_t* labels, const int64_t* act_lens,
@@ -1941,7 +1967,7 @@ int mi_rnnt_loss(const void* acts, int act_dtype, const int64_t* labels, const i
                            grads != nullptr, workspace, workspace_bytes, stream);
   if (st || !grads) return st;
   return mi_rnnt_backward(acts, act_dtype, labels, act_lens, label_lens, grads, grad_scale, grad_scale_stride,
-                          grad_mul, B, T, U, V, blank, fastemit_lambda, clamp, workspace, workspace_bytes, stream);
+                          grad_mul, 0, B, T, U, V, blank, fastemit_lambda, clamp, workspace, workspace_bytes, stream);
 }
 
 int mi_tdt_forward(const void* acts, int act_dtype, const int64_t* labels, const int64_t* act_lens,
@@ -1964,12 +1990,13 @@ int mi_tdt_forward(const void* acts, int act_dtype, const int64_t* labels, const
 
 int mi_tdt_backward(const void* acts, int act_dtype, const int64_t* labels, const int64_t* act_lens,
                     const int64_t* label_lens, void* grads, const float* grad_scale, int grad_scale_stride,
-                    float grad_mul, int B, int T, int U, int V, int D, const int32_t* durations_host, int blank,
-                    float fastemit_lambda, float clamp, float sigma, int use_plain_rnnt, void* workspace,
-                    size_t workspace_bytes, void* stream) {
+                    float grad_mul, int padding_zeroed, int B, int T, int U, int V, int D,
+                    const int32_t* durations_host, int blank, float fastemit_lambda, float clamp, float sigma,
+                    int use_plain_rnnt, void* workspace, size_t workspace_bytes, void* stream) {
   Common c;
   TdtParams prm;
   if (!grads || clamp < 0.f || grad_scale_stride < 0) return MI_TRANSDUCER_INVALID_VALUE;
+  const int pad_flag = padding_zeroed ? kFlagPaddingDone : 0;
   int st = make_tdt_params(D, durations_host, sigma, &prm);
   if (st) return st;
   st = check_common(acts, act_dtype, labels, act_lens, label_lens, B, T, U, V, D, blank, workspace, workspace_bytes,
@@ -1979,10 +2006,10 @@ int mi_tdt_backward(const void* acts, int act_dtype, const int64_t* labels, cons
   if (use_plain_rnnt) {  // gpu_rnnt.py:646-682: token gradient from the RNNT kernel, duration gradient stays zero
     const bool fused = grad_rows_R(c, grads) != 0;
     if (!fused && (st = run_rnnt_cells(c, sc, fastemit_lambda, clamp))) return st;
-    return run_grad_stream(c, grads, 1, fused, sc, fastemit_lambda, clamp);
+    return run_grad_stream(c, grads, kFlagZeroDurations | pad_flag, fused, sc, fastemit_lambda, clamp);
   }
   if ((st = run_tdt_cells(c, sc, fastemit_lambda, clamp, prm))) return st;
-  return run_grad_stream(c, grads, 0, false, sc, fastemit_lambda, clamp);
+  return run_grad_stream(c, grads, pad_flag, false, sc, fastemit_lambda, clamp);
 }
 
 int mi_tdt_loss(const void* acts, int act_dtype, const int64_t* labels, const int64_t* act_lens,
@@ -1994,7 +2021,7 @@ int mi_tdt_loss(const void* acts, int act_dtype, const int64_t* labels, const in
                           fastemit_lambda, sigma, use_plain_rnnt, grads != nullptr, workspace, workspace_bytes, stream);
   if (st || !grads) return st;
   return mi_tdt_backward(acts, act_dtype, labels, act_lens, label_lens, grads, grad_scale, grad_scale_stride, grad_mul,
-                         B, T, U, V, D, durations_host, blank, fastemit_lambda, clamp, sigma, use_plain_rnnt,
+                         0, B, T, U, V, D, durations_host, blank, fastemit_lambda, clamp, sigma, use_plain_rnnt,
                          workspace, workspace_bytes, stream);
 }
 
@@ -2018,6 +2045,65 @@ int mi_transducer_length_maxima(const int64_t* act_lens, const int64_t* label_le
                                 void* stream) {
   if (!act_lens || !label_lens || !out || B <= 0) return MI_TRANSDUCER_INVALID_VALUE;
   hipLaunchKernelGGL(length_maxima_kernel, dim3(1), dim3(256), 0, (hipStream_t)stream, act_lens, label_lens, B, out);
+  return launch_status();
+}
+
+int mi_transducer_denominators(const void* acts, int act_dtype, const int64_t* labels, const int64_t* act_lens,
+                               const int64_t* label_lens, int B, int T, int U, int V, int D, int blank,
+                               void* workspace, size_t workspace_bytes, void* stream) {
+  Common c;
+  int st = check_common(acts, act_dtype, labels, act_lens, label_lens, B, T, U, V, D, blank, workspace,
+                        workspace_bytes, stream, &c);
+  if (st) return st;
+  return run_denom(c);
+}
+
+int mi_rnnt_lattice(const int64_t* act_lens, const int64_t* label_lens, float* costs, int B, int T, int U, int D,
+                    float fastemit_lambda, int with_betas, void* workspace, size_t workspace_bytes, void* stream) {
+  Common c;
+  if (!costs || !act_lens || !label_lens || !workspace) return MI_TRANSDUCER_INVALID_VALUE;
+  if (!make_layout(B, T, U, D, &c.L) || workspace_bytes < c.L.total || ((uintptr_t)workspace & 255))
+    return MI_TRANSDUCER_INVALID_VALUE;
+  c.act_lens = act_lens; c.label_lens = label_lens;
+  c.B = B; c.T = T; c.U = U; c.D = D;
+  c.ws = (char*)workspace; c.stream = (hipStream_t)stream;
+  return run_rnnt_lattice(c, costs, fastemit_lambda, with_betas);
+}
+
+int mi_tdt_lattice(const int64_t* act_lens, const int64_t* label_lens, float* costs, int B, int T, int U, int D,
+                   const int32_t* durations_host, float fastemit_lambda, float sigma, int with_betas, void* workspace,
+                   size_t workspace_bytes, void* stream) {
+  Common c;
+  TdtParams prm;
+  if (!costs || !act_lens || !label_lens || !workspace) return MI_TRANSDUCER_INVALID_VALUE;
+  int st = make_tdt_params(D, durations_host, sigma, &prm);
+  if (st) return st;
+  if (!make_layout(B, T, U, D, &c.L) || workspace_bytes < c.L.total || ((uintptr_t)workspace & 255))
+    return MI_TRANSDUCER_INVALID_VALUE;
+  c.act_lens = act_lens; c.label_lens = label_lens;
+  c.B = B; c.T = T; c.U = U; c.D = D;
+  c.ws = (char*)workspace; c.stream = (hipStream_t)stream;
+  return run_tdt_lattice(c, costs, fastemit_lambda, with_betas, prm);
+}
+
+int mi_transducer_zero_padding(void* grads, int act_dtype, const int64_t* act_lens, const int64_t* label_lens, int B,
+                               int T, int U, int VD, void* stream) {
+  if (!grads || !act_lens || !label_lens || B <= 0 || T <= 0 || U <= 0 || VD <= 0) return MI_TRANSDUCER_INVALID_VALUE;
+  if (act_dtype != MI_DTYPE_F32 && act_dtype != MI_DTYPE_BF16 && act_dtype != MI_DTYPE_F16)
+    return MI_TRANSDUCER_INVALID_VALUE;
+  if ((long long)B * T > 65535LL * 8) return MI_TRANSDUCER_INVALID_VALUE;
+  const int nchunks = (U + kChunkRows - 1) / kChunkRows;
+  const int nblocks = nchunks * B * T;
+  const unsigned turn = 8u * MI_XCD_SPAN;
+  const dim3 grid(((unsigned)nblocks + turn - 1) / turn * turn, 1, 1);
+  ProfScope prof(MI_PROFILE_ZERO, (hipStream_t)stream);
+#define LAUNCH_ZERO(DT)                                                                                          \
+  hipLaunchKernelGGL(zero_padding_kernel<DT>, grid, dim3(kRowThreads), 0, (hipStream_t)stream, grads, act_lens,   \
+                     label_lens, T, U, VD, nchunks, nblocks)
+  if (act_dtype == MI_DTYPE_F32) LAUNCH_ZERO(MI_DTYPE_F32);
+  else if (act_dtype == MI_DTYPE_BF16) LAUNCH_ZERO(MI_DTYPE_BF16);
+  else LAUNCH_ZERO(MI_DTYPE_F16);
+#undef LAUNCH_ZERO
   return launch_status();
 }
 

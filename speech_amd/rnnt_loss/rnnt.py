@@ -79,6 +79,50 @@ def length_maxima(act_lens, label_lens):
     return out
 
 
+def zero_padding(grads, act_lens, label_lens):
+    """Zero-fill the padded cells of grads [B,T,U,V(+D)] on the CURRENT stream (nothing else is written)."""
+    _require_gpu(grads, "zero_padding")
+    B, T, U, VD = grads.shape
+    with torch.cuda.device(grads.device):
+        status = _native.lib().mi_transducer_zero_padding(
+            _ptr(grads), _dtype_code(grads), _ptr(act_lens), _ptr(label_lens), B, T, U, VD, _stream(grads.device)
+        )
+    _native.check_status(status, "zero_padding")
+
+
+def denominators(acts, labels, act_lens, label_lens, blank, workspace, num_durations=0):
+    """First stage of a forward call: log-softmax denominators and gathered arc log-probs into workspace."""
+    _require_gpu(acts, "denominators")
+    B, T, U, VD = acts.shape
+    with torch.cuda.device(acts.device):
+        status = _native.lib().mi_transducer_denominators(
+            _ptr(acts), _dtype_code(acts), _labels_ptr(labels), _ptr(act_lens), _ptr(label_lens), B, T, U,
+            VD - num_durations, num_durations, int(blank), _ptr(workspace), workspace.numel(), _stream(acts.device),
+        )  # fmt: skip
+    _native.check_status(status, "Could not calculate forward scores")
+
+
+def rnnt_lattice(act_lens, label_lens, costs, B, T, U, fastemit_lambda, with_betas, workspace, num_durations=0):
+    """Second stage: alpha (and beta) recursions and costs from what denominators() left in workspace."""
+    with torch.cuda.device(workspace.device):
+        status = _native.lib().mi_rnnt_lattice(
+            _ptr(act_lens), _ptr(label_lens), _ptr(costs), B, T, U, num_durations, float(fastemit_lambda),
+            int(bool(with_betas)), _ptr(workspace), workspace.numel(), _stream(workspace.device),
+        )  # fmt: skip
+    _native.check_status(status, "Could not calculate forward scores")
+
+
+def tdt_lattice(act_lens, label_lens, costs, B, T, U, durations, fastemit_lambda, sigma, with_betas, workspace):
+    keep, dur_ptr = _durations_array(durations)
+    with torch.cuda.device(workspace.device):
+        status = _native.lib().mi_tdt_lattice(
+            _ptr(act_lens), _ptr(label_lens), _ptr(costs), B, T, U, len(durations), dur_ptr, float(fastemit_lambda),
+            float(sigma), int(bool(with_betas)), _ptr(workspace), workspace.numel(), _stream(workspace.device),
+        )  # fmt: skip
+    del keep
+    _native.check_status(status, "Could not calculate forward scores")
+
+
 def rnnt_forward(acts, labels, act_lens, label_lens, costs, blank, fastemit_lambda, with_betas, workspace):
     _require_gpu(acts, "rnnt_forward")
     B, T, U, V = acts.shape
@@ -93,17 +137,18 @@ def rnnt_forward(acts, labels, act_lens, label_lens, costs, blank, fastemit_lamb
 
 def rnnt_backward(
     acts, labels, act_lens, label_lens, grads, grad_scale, blank, fastemit_lambda, clamp, workspace,
-    grad_scale_stride=1, grad_mul=1.0,
+    grad_scale_stride=1, grad_mul=1.0, padding_zeroed=False,
 ):  # fmt: skip
     """grad_scale: device float32 tensor read as grad_scale[b * grad_scale_stride] (or None); every gradient is
-    additionally multiplied by the host scalar grad_mul."""
+    additionally multiplied by the host scalar grad_mul.  padding_zeroed: zero_padding() already ran on grads
+    and the current stream waits for it."""
     _require_gpu(acts, "rnnt_backward")
     B, T, U, V = acts.shape
     with torch.cuda.device(acts.device):
         status = _native.lib().mi_rnnt_backward(
             _ptr(acts), _dtype_code(acts), _labels_ptr(labels), _ptr(act_lens), _ptr(label_lens), _ptr(grads),
-            _ptr(grad_scale), int(grad_scale_stride), float(grad_mul), B, T, U, V, int(blank), float(fastemit_lambda),
-            float(clamp), _ptr(workspace), workspace.numel(), _stream(acts.device),
+            _ptr(grad_scale), int(grad_scale_stride), float(grad_mul), int(bool(padding_zeroed)), B, T, U, V, int(blank),
+            float(fastemit_lambda), float(clamp), _ptr(workspace), workspace.numel(), _stream(acts.device),
         )  # fmt: skip
     _native.check_status(status, "Could not calculate gradients")
 
@@ -128,7 +173,7 @@ def tdt_forward(
 
 def tdt_backward(
     acts, labels, act_lens, label_lens, grads, grad_scale, blank, durations, fastemit_lambda, clamp, sigma,
-    use_plain_rnnt, workspace, grad_scale_stride=1, grad_mul=1.0,
+    use_plain_rnnt, workspace, grad_scale_stride=1, grad_mul=1.0, padding_zeroed=False,
 ):  # fmt: skip
     _require_gpu(acts, "tdt_backward")
     B, T, U, VD = acts.shape
@@ -137,9 +182,9 @@ def tdt_backward(
     with torch.cuda.device(acts.device):
         status = _native.lib().mi_tdt_backward(
             _ptr(acts), _dtype_code(acts), _labels_ptr(labels), _ptr(act_lens), _ptr(label_lens), _ptr(grads),
-            _ptr(grad_scale), int(grad_scale_stride), float(grad_mul), B, T, U, VD - D, D, dur_ptr, int(blank),
-            float(fastemit_lambda), float(clamp), float(sigma), int(bool(use_plain_rnnt)), _ptr(workspace),
-            workspace.numel(), _stream(acts.device),
+            _ptr(grad_scale), int(grad_scale_stride), float(grad_mul), int(bool(padding_zeroed)), B, T, U, VD - D, D,
+            dur_ptr, int(blank), float(fastemit_lambda), float(clamp), float(sigma), int(bool(use_plain_rnnt)),
+            _ptr(workspace), workspace.numel(), _stream(acts.device),
         )  # fmt: skip
     del keep
     _native.check_status(status, "Could not calculate gradients")

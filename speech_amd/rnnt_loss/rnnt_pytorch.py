@@ -20,6 +20,7 @@ What is done differently underneath:
     overlaps the forward kernels instead of two blocking torch.max calls.
 """
 
+import os
 import random
 
 import torch
@@ -29,6 +30,39 @@ from torch.nn import Module
 from speech_amd.rnnt_loss import rnnt
 
 __all__ = ['RNNTLossNumba', 'TDTLossNumba', 'RNNTLossMI355X', 'TDTLossMI355X', 'certify_inputs']
+
+
+# When the gradient will be needed, forward allocates it and, once the denominators are done,
+# zero-fills its padded cells on a second stream: that part of the gradient depends on the lengths
+# only, and HBM would otherwise idle while the lattice recursion (and the small kernels between
+# forward and backward) run.  Backward writes the valid cells beside whatever is left of the fill
+# (disjoint bytes) and joins the two streams.  MI_TRANSDUCER_OVERLAP=0 turns this off: backward
+# then allocates the gradient and writes all of it in one pass.
+OVERLAP_PADDING = os.environ.get("MI_TRANSDUCER_OVERLAP", "1") != "0"
+
+_aux_streams = {}
+
+
+def _aux_stream(device):
+    stream = _aux_streams.get(device.index)
+    if stream is None:
+        stream = torch.cuda.Stream(device=device)  # default priority
+        _aux_streams[device.index] = stream
+    return stream
+
+
+def _start_padding_fill(grads, act_lens, label_lens):
+    """Enqueue the zero-fill of the padded cells of grads on the auxiliary stream, ordered after
+    everything enqueued so far on the current stream.  Returns the event recorded after the fill."""
+    main = torch.cuda.current_stream(grads.device)
+    aux = _aux_stream(grads.device)
+    aux.wait_stream(main)
+    with torch.cuda.stream(aux):
+        rnnt.zero_padding(grads, act_lens, label_lens)
+        done = torch.cuda.Event()
+        done.record(aux)
+    grads.record_stream(aux)
+    return done
 
 
 def check_type(var, t, name):
@@ -158,7 +192,15 @@ class _RNNTNumba(Function):
         batch = acts.size(0)
         costs = torch.empty(batch, device=acts.device, dtype=torch.float32)
         workspace = rnnt.new_workspace(acts)
-        rnnt.rnnt_forward(acts, labels, act_lens, label_lens, costs, blank, fastemit_lambda, need_grad, workspace)
+        ctx.padding = None
+        if need_grad and OVERLAP_PADDING:
+            grads = torch.empty_like(acts)
+            rnnt.denominators(acts, labels, act_lens, label_lens, blank, workspace)
+            ctx.padding = (grads, _start_padding_fill(grads, act_lens, label_lens))
+            B, T, U = acts.shape[:3]
+            rnnt.rnnt_lattice(act_lens, label_lens, costs, B, T, U, fastemit_lambda, True, workspace)
+        else:
+            rnnt.rnnt_forward(acts, labels, act_lens, label_lens, costs, blank, fastemit_lambda, need_grad, workspace)
         pending.finish()  # raises ValueError exactly where certify_inputs would
 
         costs = _reduce_costs(costs, reduction, batch)
@@ -171,11 +213,15 @@ class _RNNTNumba(Function):
     def backward(ctx, grad_output):
         acts, labels, act_lens, label_lens, workspace = ctx.saved_tensors
         blank, reduction, fastemit_lambda, clamp = ctx.params
-        grads = torch.empty_like(acts)
+        prepared, ctx.padding = ctx.padding, None  # the prepared buffer serves the first backward call only
+        grads = prepared[0] if prepared else torch.empty_like(acts)
         scale, stride, mul = _grad_scale(grad_output, reduction, acts.size(0), acts.device)
         rnnt.rnnt_backward(
-            acts, labels, act_lens, label_lens, grads, scale, blank, fastemit_lambda, clamp, workspace, stride, mul
-        )
+            acts, labels, act_lens, label_lens, grads, scale, blank, fastemit_lambda, clamp, workspace, stride, mul,
+            prepared is not None,
+        )  # fmt: skip
+        if prepared:
+            torch.cuda.current_stream(acts.device).wait_event(prepared[1])  # join the padding fill
         return grads, None, None, None, None, None, None, None
 
 
@@ -204,10 +250,22 @@ class _TDTNumba(Function):
         workspace = rnnt.new_workspace(acts, len(durations))
         # gpu_rnnt.py:606-607: one host-side draw per call decides between the TDT and the plain RNNT kernels
         use_plain_rnnt = random.uniform(0, 1) < omega
-        rnnt.tdt_forward(
-            acts, labels, act_lens, label_lens, costs, blank, durations, fastemit_lambda, sigma, use_plain_rnnt,
-            need_grad, workspace,
-        )  # fmt: skip
+        ctx.padding = None
+        if need_grad and OVERLAP_PADDING:
+            grads = torch.empty_like(acts)
+            D = len(durations)
+            rnnt.denominators(acts, labels, act_lens, label_lens, blank, workspace, D)
+            ctx.padding = (grads, _start_padding_fill(grads, act_lens, label_lens))
+            B, T, U = acts.shape[:3]
+            if use_plain_rnnt:
+                rnnt.rnnt_lattice(act_lens, label_lens, costs, B, T, U, fastemit_lambda, True, workspace, D)
+            else:
+                rnnt.tdt_lattice(act_lens, label_lens, costs, B, T, U, durations, fastemit_lambda, sigma, True, workspace)
+        else:
+            rnnt.tdt_forward(
+                acts, labels, act_lens, label_lens, costs, blank, durations, fastemit_lambda, sigma, use_plain_rnnt,
+                need_grad, workspace,
+            )  # fmt: skip
         pending.finish()
 
         # the reference allocates TDT costs in the dtype of acts (rnnt_pytorch.py:145)
@@ -221,12 +279,15 @@ class _TDTNumba(Function):
     def backward(ctx, grad_output):
         acts, labels, act_lens, label_lens, workspace = ctx.saved_tensors
         blank, durations, reduction, fastemit_lambda, clamp, sigma, use_plain_rnnt = ctx.params
-        grads = torch.empty_like(acts)
+        prepared, ctx.padding = ctx.padding, None
+        grads = prepared[0] if prepared else torch.empty_like(acts)
         scale, stride, mul = _grad_scale(grad_output, reduction, acts.size(0), acts.device)
         rnnt.tdt_backward(
             acts, labels, act_lens, label_lens, grads, scale, blank, durations, fastemit_lambda, clamp, sigma,
-            use_plain_rnnt, workspace, stride, mul,
+            use_plain_rnnt, workspace, stride, mul, prepared is not None,
         )  # fmt: skip
+        if prepared:
+            torch.cuda.current_stream(acts.device).wait_event(prepared[1])
         return grads, None, None, None, None, None, None, None, None, None, None
 
 

@@ -111,7 +111,9 @@ def algorithmic_bytes(cfg, act_lens, label_lens):
     return dict(
         total=2 * c_valid * width * s + cells * width * s + 24 * c_valid,
         denom_gather=c_valid * width * s + 12 * c_valid,
-        grad_stream=c_valid * width * s + cells * width * s,
+        grad_stream=c_valid * width * s + cells * width * s,  # gradient pass that also zero-fills the padding
+        grad_valid=2 * c_valid * width * s,  # gradient pass over the valid rows only
+        zero_padding=(cells - c_valid) * width * s,
         c_valid=c_valid,
         cells=cells,
     )
