@@ -514,6 +514,9 @@ __global__ __launch_bounds__(64) void rnnt_lattice_kernel(const float* __restric
                                                           int A, float cost_scale, int with_betas) {
   constexpr int P = Prefetch<K>::P;
   constexpr int Us = 64 * K;
+  // the recursion is one long dependent chain: let this wave win the issue arbitration against
+  // whatever bandwidth-bound waves share its SIMD
+  __builtin_amdgcn_s_setprio(3);
   const int b = with_betas ? (int)(blockIdx.x >> 1) : (int)blockIdx.x;
   const int dir = with_betas ? (int)(blockIdx.x & 1) : 0;
   const int lane = threadIdx.x;
