@@ -32,13 +32,13 @@ from speech_amd.rnnt_loss import rnnt
 __all__ = ['RNNTLossNumba', 'TDTLossNumba', 'RNNTLossMI355X', 'TDTLossMI355X', 'certify_inputs']
 
 
-# When the gradient will be needed, forward allocates it and, once the denominators are done,
-# zero-fills its padded cells on a second stream: that part of the gradient depends on the lengths
-# only, and HBM would otherwise idle while the lattice recursion (and the small kernels between
-# forward and backward) run.  Backward writes the valid cells beside whatever is left of the fill
-# (disjoint bytes) and joins the two streams.  MI_TRANSDUCER_OVERLAP=0 turns this off: backward
-# then allocates the gradient and writes all of it in one pass.
-OVERLAP_PADDING = os.environ.get("MI_TRANSDUCER_OVERLAP", "1") != "0"
+# Optional (MI_TRANSDUCER_OVERLAP=1): when the gradient will be needed, forward allocates it and,
+# once the denominators are done, zero-fills its padded cells on a second stream while the lattice
+# recursion runs; backward then writes the valid cells only and joins the two streams.  Off by
+# default: the recursion is a chain of dependent memory round trips, and a fill that saturates HBM
+# beside it stretches every step of the chain, so the measured step time is no better than with
+# backward writing the whole gradient in one pass.
+OVERLAP_PADDING = os.environ.get("MI_TRANSDUCER_OVERLAP", "0") == "1"
 
 _aux_streams = {}
 
