@@ -26,6 +26,7 @@
 
 #include <hip/hip_runtime.h>
 #include <math.h>
+#include <string.h>
 #include <stdint.h>
 
 #include <vector>
@@ -312,6 +313,36 @@ template <int DT> struct RowSplit {
     return -1;
   }
 };
+
+// A load through the scalar unit: for a wave-uniform address of data that no store of the running
+// kernel touches (inputs, and what earlier kernels of the stream left in the workspace).  Scalar
+// loads do not queue behind the wave's vector traffic.
+template <class T> __device__ __forceinline__ T sload(const T* p) {
+  typedef const T __attribute__((address_space(4))) * const_ptr;
+  return *(const_ptr)(unsigned long long)p;
+}
+// wave-uniform values as the compiler should see them: held in scalar registers
+__device__ __forceinline__ int uni(int v) { return __builtin_amdgcn_readfirstlane(v); }
+__device__ __forceinline__ float uni(float v) { return __int_as_float(uni(__float_as_int(v))); }
+__device__ __forceinline__ double uni(double v) {
+  return __hiloint2double(uni(__double2hiint(v)), uni(__double2loint(v)));
+}
+__device__ __forceinline__ long long uni(long long v) {
+  const unsigned lo = (unsigned)uni((int)(unsigned)v), hi = (unsigned)uni((int)((unsigned long long)v >> 32));
+  return (long long)(((unsigned long long)hi << 32) | lo);
+}
+// the two lengths of utterance b, clamped into the tensor, fetched in one round trip
+struct UttLens {
+  int Tb, Ub;
+};
+__device__ __forceinline__ UttLens load_lens(const int64_t* act_lens, const int64_t* label_lens, int b, int T, int U) {
+  long long len_t = uni((long long)sload(act_lens + b)), len_u = uni((long long)sload(label_lens + b));
+  asm("" : "+s"(len_t), "+s"(len_u));
+  UttLens r;
+  r.Tb = clampi(len_t, 1, T);
+  r.Ub = clampi(len_u + 1, 1, U);
+  return r;
+}
 
 // running (max, sum of exp) of one lane, base-2 scaled: sum_i 2^(x_i*log2e - m*log2e)
 struct LaneLse {
@@ -1023,6 +1054,62 @@ __device__ __forceinline__ RowCoef rnnt_coef(const float* __restrict__ denom, co
   return make_coef(dn, gamma + lambda * pl, pb, (1.f + lambda) * pl, lpb, lpl, lab, blank, clamp, scale);
 }
 
+// The same coefficients for a wave that works on one row (every input is wave-uniform).  The ten
+// values are fetched by scalar loads that are all issued before the first of them is awaited: a
+// load placed under the condition that uses it would cost one memory round trip per condition.
+struct CoefRaw {
+  double a, bb, b_down, b_right, L;
+  float lpb, lpl, dn, gs;
+  long long lab;
+};
+__device__ __forceinline__ CoefRaw load_coef_raw_from(const float* __restrict__ denom, const float* __restrict__ arcs,
+                                                      const double* __restrict__ alphas,
+                                                      const double* __restrict__ betas, const double* __restrict__ ll,
+                                                      const int64_t* __restrict__ labels,
+                                                      const float* __restrict__ grad_scale, int grad_scale_stride,
+                                                      int ND, int Us, int A, int b, int t, int u, int Tb, int Ub,
+                                                      int T, int U) {
+  const size_t row = (size_t)(b * ND + t + u);
+  const size_t sk = row * Us + u;
+  const bool has_down = t < Tb - 1, has_lab = u < Ub - 1;
+  // a row without a label arc (and U == 1, where there is no label array at all) reads a dummy word
+  const int64_t* lp = has_lab ? labels + ((size_t)b * (U - 1) + u) : (const int64_t*)ll;
+  const float* gp = grad_scale ? grad_scale + (size_t)b * grad_scale_stride : (const float*)ll;
+  CoefRaw r;
+  r.a = uni(sload(alphas + sk));
+  r.bb = uni(sload(betas + sk));
+  r.b_down = uni(sload(betas + sk + (has_down ? Us : 0)));      // beta(t+1,u): next diagonal, same column
+  r.b_right = uni(sload(betas + sk + (has_lab ? Us + 1 : 0)));  // beta(t,u+1)
+  r.L = uni(sload(ll + 2 * b));
+  r.lpb = uni(sload(arcs + row * A * Us + u));
+  r.lpl = uni(sload(arcs + row * A * Us + Us + u));
+  r.dn = uni(sload(denom + ((size_t)b * T + t) * U + u));
+  r.lab = uni((long long)sload(lp));
+  r.gs = uni(sload(gp));
+  // every value is now on its way; the registers are claimed here, before any of them is used
+  // (an asm without side effects: one that has them would turn every later load into a vector load)
+  asm("" : "+s"(r.a), "+s"(r.bb), "+s"(r.b_down), "+s"(r.b_right), "+s"(r.L), "+s"(r.lpb), "+s"(r.lpl), "+s"(r.dn),
+      "+s"(r.gs), "+s"(r.lab));
+  return r;
+}
+__device__ __forceinline__ CoefRaw load_coef_raw(const LatticeView& lv, int b, int t, int u, int Tb, int Ub, int T,
+                                                 int U) {
+  return load_coef_raw_from(lv.denom, lv.arcs, lv.alphas, lv.betas, lv.ll, lv.labels, lv.grad_scale,
+                            lv.grad_scale_stride, lv.ND, lv.Us, lv.A, b, t, u, Tb, Ub, T, U);
+}
+__device__ __forceinline__ RowCoef finish_coef(const CoefRaw& r, const LatticeView& lv, int t, int u, int Tb, int Ub,
+                                               int V, int blank) {
+  const int lab = (u < Ub - 1) ? clampi(r.lab, 0, V - 1) : -1;
+  const float scale = (lv.grad_scale ? r.gs : 1.f) * lv.grad_mul;
+  const float gamma = __expf((float)(r.a + r.bb - r.L));
+  float pb = 0.f, pl = 0.f;
+  if (t < Tb - 1) pb = __expf((float)(r.a + r.b_down - r.L + (double)r.lpb));
+  else if (u == Ub - 1) pb = __expf((float)(r.a - r.L + (double)r.lpb));
+  if (lab >= 0) pl = __expf((float)(r.a + r.b_right - r.L + (double)r.lpl));
+  return make_coef(r.dn, gamma + lv.lambda * pl, pb, (1.f + lv.lambda) * pl, r.lpb, r.lpl, lab, blank, lv.clamp,
+                   scale);
+}
+
 __global__ __launch_bounds__(256) void rnnt_cell_kernel(
     const float* __restrict__ denom, const float* __restrict__ arcs, const double* __restrict__ alphas,
     const double* __restrict__ betas, const double* __restrict__ ll, const int64_t* __restrict__ labels,
@@ -1288,6 +1375,11 @@ __global__ __launch_bounds__(kRowThreads) void denom_rows_kernel(
     const int64_t* __restrict__ label_lens, float* __restrict__ denom, float* __restrict__ arcs, int T, int U, int V,
     int D, int blank, int ND, int Us, int A, int nchunks, int nblocks) {
   constexpr int VEC = Elem<DT>::VEC;
+  // all kernel arguments are fetched in one go, not one batch per use (the loads this kernel wants
+  // on the scalar unit are written as such, so the asm's side effect costs nothing)
+  asm volatile("" ::"s"((uintptr_t)acts), "s"((uintptr_t)labels), "s"((uintptr_t)act_lens), "s"((uintptr_t)label_lens),
+               "s"((uintptr_t)denom), "s"((uintptr_t)arcs), "s"(T), "s"(U), "s"(V), "s"(D), "s"(blank), "s"(ND), "s"(Us),
+               "s"(A), "s"(nchunks), "s"(nblocks));
   const int lane = threadIdx.x & 63;
   const int wave = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
   // 1-D grid over (b,t,chunk), chunk fastest = memory order
@@ -1298,10 +1390,20 @@ __global__ __launch_bounds__(kRowThreads) void denom_rows_kernel(
 #endif
   const unsigned bt = wg / (unsigned)nchunks, chunk = wg - bt * (unsigned)nchunks;
   const int b = (int)(bt / (unsigned)T), t = (int)(bt - (unsigned)b * (unsigned)T);
-  const int Tb = clampi(act_lens[b], 1, T);
-  const int Ub = clampi(label_lens[b] + 1, 1, U);
-  if (t >= Tb) return;
   const int u_begin = (int)chunk * kChunkRows + wave;
+  // the wave's label ids travel with the lengths (a clamped index, dropped below if the row has no
+  // label arc; with U == 1 there is no label array and a length is read instead)
+  long long lab_raw[kRowsPerWave];
+#pragma unroll
+  for (int i = 0; i < kRowsPerWave; ++i) {
+    const int uu = min(u_begin + kRowWaves * i, U - 2);
+    lab_raw[i] = uni((long long)sload(U > 1 ? labels + ((size_t)b * (U - 1) + max(uu, 0)) : act_lens + b));
+  }
+  const UttLens len = load_lens(act_lens, label_lens, b, T, U);
+#pragma unroll
+  for (int i = 0; i < kRowsPerWave; ++i) asm("" : "+s"(lab_raw[i]));
+  const int Tb = len.Tb, Ub = len.Ub;
+  if (t >= Tb) return;
   const int u_end = min(Ub, (int)(chunk + 1) * kChunkRows);
   if (u_begin >= u_end) return;
   const int VD = V + D;
@@ -1312,7 +1414,7 @@ __global__ __launch_bounds__(kRowThreads) void denom_rows_kernel(
 #pragma unroll
   for (int i = 0; i < kRowsPerWave; ++i) {
     const int uu = u_begin + kRowWaves * i;
-    labs[i] = (uu < Ub - 1) ? clampi(labels[(size_t)b * (U - 1) + uu], 0, V - 1) : -1;
+    labs[i] = (uu < Ub - 1) ? clampi(lab_raw[i], 0, V - 1) : -1;
   }
 
   struct Row {
@@ -1406,6 +1508,14 @@ __global__ __launch_bounds__(kRowThreads) void grad_rows_kernel(const void* __re
                                                         int D, int blank, int CS, int flags, int nchunks,
                                                         int nblocks) {
   constexpr int VEC = Elem<DT>::VEC;
+  // all kernel arguments are fetched in one go, not one batch per use (the loads this kernel wants
+  // on the scalar unit are written as such, so the asm's side effect costs nothing)
+  asm volatile("" ::"s"((uintptr_t)acts), "s"((uintptr_t)grads), "s"((uintptr_t)coef), "s"((uintptr_t)act_lens),
+               "s"((uintptr_t)label_lens), "s"((uintptr_t)lv.denom), "s"((uintptr_t)lv.arcs), "s"((uintptr_t)lv.alphas),
+               "s"((uintptr_t)lv.betas), "s"((uintptr_t)lv.ll), "s"((uintptr_t)lv.labels), "s"((uintptr_t)lv.grad_scale),
+               "s"(lv.grad_scale_stride), "s"(lv.grad_mul), "s"(lv.ND), "s"(lv.Us), "s"(lv.A), "s"(lv.lambda),
+               "s"(lv.clamp), "s"(T), "s"(U), "s"(V), "s"(D), "s"(blank), "s"(CS), "s"(flags), "s"(nchunks),
+               "s"(nblocks));
   const int lane = threadIdx.x & 63;
   const int wave = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
   // 1-D grid over (b,t,chunk), chunk fastest = memory order
@@ -1416,8 +1526,8 @@ __global__ __launch_bounds__(kRowThreads) void grad_rows_kernel(const void* __re
 #endif
   const unsigned bt = wg / (unsigned)nchunks, chunk = wg - bt * (unsigned)nchunks;
   const int b = (int)(bt / (unsigned)T), t = (int)(bt - (unsigned)b * (unsigned)T);
-  const int Tb = clampi(act_lens[b], 1, T);
-  const int Ub = clampi(label_lens[b] + 1, 1, U);
+  const UttLens len = load_lens(act_lens, label_lens, b, T, U);
+  const int Tb = len.Tb, Ub = len.Ub;
   const int VD = V + D;
   const size_t cell0 = ((size_t)b * T + t) * U;
   const int c0 = (int)chunk * kChunkRows;
@@ -1427,8 +1537,6 @@ __global__ __launch_bounds__(kRowThreads) void grad_rows_kernel(const void* __re
   if (!(flags & kFlagPaddingDone)) zero_elems<DT>(grads, (cell0 + z0) * VD, (cell0 + c1) * VD);
   const int u_begin = c0 + wave;
   if (u_begin >= z0) return;
-  float scale = 1.f;
-  if constexpr (FUSED) scale = (lv.grad_scale ? lv.grad_scale[(size_t)b * lv.grad_scale_stride] : 1.f) * lv.grad_mul;
 
   struct Row {
     uint4 raw[R];
@@ -1453,8 +1561,8 @@ __global__ __launch_bounds__(kRowThreads) void grad_rows_kernel(const void* __re
     const int v = extra_index(sp);
     d.xe = Elem<DT>::load1(acts, e0 + ((v >= 0 && v < V) ? v : blank));
     if constexpr (FUSED) {
-      d.c = rnnt_coef(lv.denom, lv.arcs, lv.alphas, lv.betas, lv.ll, lv.labels, scale, b, t, uu, Tb, Ub, T, U, V, blank,
-                      lv.ND, lv.Us, lv.A, lv.lambda, lv.clamp);
+      const CoefRaw cr = load_coef_raw(lv, b, t, uu, Tb, Ub, T, U);
+      d.c = finish_coef(cr, lv, t, uu, Tb, Ub, V, blank);
       d.gd = 0.f;
     } else {
       const float* c = coef + (cell0 + uu) * CS;
@@ -1541,6 +1649,234 @@ __global__ __launch_bounds__(kRowThreads) void zero_padding_kernel(void* __restr
   const int c1 = min(U, c0 + kChunkRows);
   const int z0 = (t >= Tb) ? c0 : max(c0, min(Ub, c1));
   zero_elems<DT>(grads, (cell0 + z0) * VD, (cell0 + c1) * VD);
+}
+
+// ----------------------------------------------------------------------------------------
+// The bandwidth passes for rows too long to sit in one wave's registers: a workgroup of RT
+// threads owns one row, every thread moves NVT aligned 16-byte vectors (RT apart), and the
+// waves' partial (max, sum) pairs meet in LDS.  Wave 0 of a row also moves the row's ragged
+// head and tail (and the duration entries of a TDT row), one element per lane.
+// ----------------------------------------------------------------------------------------
+template <int RT> struct BlockRows {
+  static constexpr int THREADS = RT < 256 ? 256 : RT;
+  static constexpr int ROWS = THREADS / RT;  // rows per workgroup
+  static constexpr int WPR = RT / 64;        // waves per row
+};
+
+template <int DT, int RT, int NVT>
+__global__ __launch_bounds__(BlockRows<RT>::THREADS) void denom_block_kernel(
+    const void* __restrict__ acts, const int64_t* __restrict__ labels, const int64_t* __restrict__ act_lens,
+    const int64_t* __restrict__ label_lens, float* __restrict__ denom, float* __restrict__ arcs, int T, int U, int V,
+    int D, int blank, int ND, int Us, int A, int nchunks, int nblocks) {
+  constexpr int VEC = Elem<DT>::VEC;
+  constexpr int ROWS = BlockRows<RT>::ROWS, WPR = BlockRows<RT>::WPR, WAVES = BlockRows<RT>::THREADS / 64;
+  __shared__ float2 part[WAVES];
+  // all kernel arguments are fetched in one go, not one batch per use (the loads this kernel wants
+  // on the scalar unit are written as such, so the asm's side effect costs nothing)
+  asm volatile("" ::"s"((uintptr_t)acts), "s"((uintptr_t)labels), "s"((uintptr_t)act_lens), "s"((uintptr_t)label_lens),
+               "s"((uintptr_t)denom), "s"((uintptr_t)arcs), "s"(T), "s"(U), "s"(V), "s"(D), "s"(blank), "s"(ND), "s"(Us),
+               "s"(A), "s"(nchunks), "s"(nblocks));
+  const int lane = threadIdx.x & 63;
+  const int wave = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
+  const int row_in_wg = wave / WPR, wave_in_row = wave - row_in_wg * WPR;
+  const int tr = wave_in_row * 64 + lane;  // thread within the row
+  unsigned wg = logical_block();
+  if (wg >= (unsigned)nblocks) return;
+#if MI_K1_REVERSE
+  wg = (unsigned)nblocks - 1u - wg;
+#endif
+  const unsigned bt = wg / (unsigned)nchunks, chunk = wg - bt * (unsigned)nchunks;
+  const int b = (int)(bt / (unsigned)T), t = (int)(bt - (unsigned)b * (unsigned)T);
+  const int u = (int)chunk * ROWS + row_in_wg;
+  // the row's label id travels with the lengths (a clamped index, dropped below if the row has no
+  // label arc; with U == 1 there is no label array and a length is read instead)
+  long long lab_raw = uni((long long)sload(U > 1 ? labels + ((size_t)b * (U - 1) + max(min(u, U - 2), 0)) : act_lens + b));
+  const UttLens len = load_lens(act_lens, label_lens, b, T, U);
+  asm("" : "+s"(lab_raw));
+  const int Tb = len.Tb, Ub = len.Ub;
+  if (t >= Tb || (int)chunk * ROWS >= Ub) return;  // the whole workgroup leaves: no barrier is left waiting
+  const bool live = u < Ub;  // wave-uniform
+  const int VD = V + D;
+  const size_t cell0 = ((size_t)b * T + t) * U;
+  const size_t e0 = (cell0 + (live ? u : 0)) * VD;
+
+  float m_w = -1.0e30f, s_w = 0.f;  // this wave's share of the row: max and sum of 2^((x - max) log2 e)
+  float xb = 0.f, xl = 0.f, xd = 0.f;
+  int lab = -1;
+  if (live) {
+    const RowWindow<DT> w(acts, e0);
+    const RowSplit<DT> sp(w.mis, V);
+    uint4 raw[NVT];
+#pragma unroll
+    for (int k = 0; k < NVT; ++k) raw[k] = load_stream<MI_NT_K1 != 0>(w.vp + sp.body_vector(tr + RT * k));
+    float xe = kNegInf;
+    if (wave_in_row == 0) {
+      lab = (u < Ub - 1) ? clampi(lab_raw, 0, V - 1) : -1;
+      const int ve = sp.extra_token(lane);
+      const float x1 = Elem<DT>::load1(acts, e0 + (ve >= 0 ? ve : blank));
+      xb = Elem<DT>::load1(acts, e0 + blank);
+      xl = Elem<DT>::load1(acts, e0 + (lab >= 0 ? lab : blank));
+      xd = Elem<DT>::load1(acts, e0 + (lane < D ? V + lane : blank));
+      xe = ve >= 0 ? x1 : kNegInf;
+    }
+    float x[NVT][VEC];
+#pragma unroll
+    for (int k = 0; k < NVT; ++k) {
+      Elem<DT>::unpack(raw[k], x[k]);
+      const bool ok = tr + RT * k < sp.nb;
+#pragma unroll
+      for (int i = 0; i < VEC; ++i) x[k][i] = ok ? x[k][i] : kNegInf;
+    }
+    float cm = xe;
+#pragma unroll
+    for (int k = 0; k < NVT; ++k)
+#pragma unroll
+      for (int i = 0; i < VEC; ++i) cm = fmaxf(cm, x[k][i]);
+    m_w = fmaxf(wave_max_u(cm), -1.0e30f);  // finite even for a wave that holds no element of the row
+    const float off = -m_w * kLog2e;
+    float acc = stream_exp2(fmaf(xe, kLog2e, off));
+#pragma unroll
+    for (int k = 0; k < NVT; ++k)
+#pragma unroll
+      for (int i = 0; i < VEC; ++i) acc += stream_exp2(fmaf(x[k][i], kLog2e, off));
+    s_w = wave_sum_u(acc);
+  }
+  if (lane == 0) part[wave] = make_float2(m_w, s_w);
+  __syncthreads();
+  if (!live || wave_in_row != 0) return;
+  float M = -1.0e30f;
+#pragma unroll
+  for (int i = 0; i < WPR; ++i) M = fmaxf(M, part[row_in_wg * WPR + i].x);
+  float S = 0.f;
+#pragma unroll
+  for (int i = 0; i < WPR; ++i) {
+    const float2 p = part[row_in_wg * WPR + i];
+    S = fmaf(p.y, fast_exp2((p.x - M) * kLog2e), S);
+  }
+  const float dn = -M - __builtin_amdgcn_logf(S) * 0.6931471805599453f;
+  const size_t base = ((size_t)(b * ND + t + u) * A) * Us + u;
+  if (lane == 0) {
+    denom[cell0 + u] = dn;
+    arcs[base] = xb + dn;
+    arcs[base + Us] = lab >= 0 ? xl + dn : 0.f;
+  }
+  if (D > 0) {  // duration log-softmax (rnnt_pytorch.py:568), one lane per duration
+    const float xdm = lane < D ? xd : kNegInf;
+    const float dm = wave_max_u(xdm);
+    const float ds = wave_sum_u(lane < D ? expf(xdm - dm) : 0.f);
+    const float dden = -dm - logf(ds);
+    if (lane < D) arcs[base + (size_t)(2 + lane) * Us] = xdm + dden;
+  }
+}
+
+template <int DT, int RT, int NVT, bool FUSED>
+__global__ __launch_bounds__(BlockRows<RT>::THREADS) void grad_block_kernel(
+    const void* __restrict__ acts, void* __restrict__ grads, const float* __restrict__ coef, LatticeView lv,
+    const int64_t* __restrict__ act_lens, const int64_t* __restrict__ label_lens, int T, int U, int V, int D,
+    int blank, int CS, int flags, int nchunks, int nblocks) {
+  constexpr int VEC = Elem<DT>::VEC;
+  constexpr int ROWS = BlockRows<RT>::ROWS, WPR = BlockRows<RT>::WPR;
+  // all kernel arguments are fetched in one go, not one batch per use (the loads this kernel wants
+  // on the scalar unit are written as such, so the asm's side effect costs nothing)
+  asm volatile("" ::"s"((uintptr_t)acts), "s"((uintptr_t)grads), "s"((uintptr_t)coef), "s"((uintptr_t)act_lens),
+               "s"((uintptr_t)label_lens), "s"((uintptr_t)lv.denom), "s"((uintptr_t)lv.arcs), "s"((uintptr_t)lv.alphas),
+               "s"((uintptr_t)lv.betas), "s"((uintptr_t)lv.ll), "s"((uintptr_t)lv.labels), "s"((uintptr_t)lv.grad_scale),
+               "s"(lv.grad_scale_stride), "s"(lv.grad_mul), "s"(lv.ND), "s"(lv.Us), "s"(lv.A), "s"(lv.lambda),
+               "s"(lv.clamp), "s"(T), "s"(U), "s"(V), "s"(D), "s"(blank), "s"(CS), "s"(flags), "s"(nchunks),
+               "s"(nblocks));
+  const int lane = threadIdx.x & 63;
+  const int wave = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
+  const int row_in_wg = wave / WPR, wave_in_row = wave - row_in_wg * WPR;
+  const int tr = wave_in_row * 64 + lane;
+  unsigned wg = logical_block();
+  if (wg >= (unsigned)nblocks) return;
+#if MI_K4_REVERSE
+  wg = (unsigned)nblocks - 1u - wg;
+#endif
+  const unsigned bt = wg / (unsigned)nchunks, chunk = wg - bt * (unsigned)nchunks;
+  const int b = (int)(bt / (unsigned)T), t = (int)(bt - (unsigned)b * (unsigned)T);
+  const int u = (int)chunk * ROWS + row_in_wg;
+  if (u >= U) return;
+  const UttLens len = load_lens(act_lens, label_lens, b, T, U);
+  const int Tb = len.Tb, Ub = len.Ub;
+  const int VD = V + D;
+  const size_t cell0 = ((size_t)b * T + t) * U;
+  const size_t e0 = (cell0 + u) * VD;
+  const RowWindow<DT> w(acts, e0);
+  const RowSplit<DT> sp(w.mis, V);
+  char* grow = (char*)grads + e0 * Elem<DT>::BYTES;  // same 16-byte phase as the acts row
+  uint4* gvp = (uint4*)(grow - w.mis * Elem<DT>::BYTES) + sp.jb0 + tr;
+  // head, tail and duration entries of a row: one element per lane of the row's wave 0
+  int v = -1;
+  if (wave_in_row == 0) {
+    v = sp.extra_token(lane);
+    if (lane >= 2 * VEC && lane < 2 * VEC + D) v = V + lane - 2 * VEC;
+  }
+
+  if (t >= Tb || u >= Ub) {  // a padded row: zeros
+    if (flags & kFlagPaddingDone) return;
+    const uint4 z = make_uint4(0, 0, 0, 0);
+#pragma unroll
+    for (int k = 0; k < NVT; ++k)
+      if (tr + RT * k < sp.nb) store_stream(gvp + RT * k, z);
+    if (v >= 0) Elem<DT>::store1(grads, e0 + v, 0.f);
+    return;
+  }
+
+  uint4 raw[NVT];
+#pragma unroll
+  for (int k = 0; k < NVT; ++k) raw[k] = load_stream<MI_NT_K4 != 0>(w.vp + sp.body_vector(tr + RT * k));
+  float xe = 0.f, gd = 0.f;
+  if (wave_in_row == 0) xe = Elem<DT>::load1(acts, e0 + ((v >= 0 && v < V) ? v : blank));
+  RowCoef c;
+  if constexpr (FUSED) {
+    const CoefRaw cr = load_coef_raw(lv, b, t, u, Tb, Ub, T, U);
+    c = finish_coef(cr, lv, t, u, Tb, Ub, V, blank);
+  } else {
+    const float* cp = coef + (cell0 + u) * CS;
+    const float4 ca = *(const float4*)cp;        // denom*log2e, W*scale, clamp bound, G_blank
+    const float2 cb = *(const float2*)(cp + 4);  // G_label, label id
+    c.dl2 = ca.x; c.W = ca.y; c.cb = ca.z; c.gB = ca.w; c.gL = cb.x;
+    c.lab = __float_as_int(cb.y);
+    if (wave_in_row == 0) gd = cp[v >= V ? kCoefBase + v - V : 0];
+  }
+  const float dl2 = c.dl2, W = c.W, cbnd = c.cb, gB = c.gB, gL = c.gL;
+  const int lab = c.lab;
+  const bool clamp_on = cbnd < INFINITY;
+  const int jblank = (blank + w.mis) / VEC - sp.jb0, jlab = lab >= 0 ? (lab + w.mis) / VEC - sp.jb0 : -1;
+#pragma unroll
+  for (int k = 0; k < NVT; ++k) {
+    const int j = tr + RT * k;  // whole vector j of the row
+    if (j < sp.nb) {
+      float x[VEC], g[VEC];
+      Elem<DT>::unpack(raw[k], x);
+#pragma unroll
+      for (int i = 0; i < VEC; ++i) {
+        float gi = stream_exp2(fmaf(x[i], kLog2e, dl2)) * W;
+        if (clamp_on) gi = clamp_sym(gi, cbnd);
+        g[i] = gi;
+      }
+      if (j == jblank || j == jlab) {  // the two special logits are patched in the vector that holds them
+        const int first = sp.hc + j * VEC;
+#pragma unroll
+        for (int i = 0; i < VEC; ++i) {
+          if (first + i == blank) g[i] = gB;
+          if (first + i == lab) g[i] = gL;
+        }
+      }
+      store_stream(gvp + RT * k, Elem<DT>::pack(g));
+    }
+  }
+  if (v >= 0) {
+    float g = (flags & kFlagZeroDurations) ? 0.f : gd;
+    if (v < V) {
+      g = stream_exp2(fmaf(xe, kLog2e, dl2)) * W;
+      if (clamp_on) g = clamp_sym(g, cbnd);
+      if (v == blank) g = gB;
+      if (v == lab) g = gL;
+    }
+    Elem<DT>::store1(grads, e0 + v, g);
+  }
 }
 
 // ----------------------------------------------------------------------------------------
@@ -1722,6 +2058,64 @@ inline int grad_rows_R(const Common& c, const void* grads) {
   const bool same_phase = (((uintptr_t)c.acts ^ (uintptr_t)grads) & 15) == 0;
   return same_phase ? rows_R(c) : 0;
 }
+// Workgroup-per-row kernels: RT threads per row, NVT vectors per thread.  RT == 0: not applicable.
+// The denominator pass uses them for rows too long for the register-resident wave-per-row
+// kernels (more than 512 whole vectors).  The gradient pass uses them from 65 vectors up, with
+// two vectors per thread where the row allows it: of the splits tried (1, 2 and 4 vectors per
+// thread) that one streams fastest.
+#ifndef MI_USE_BLOCK_ROWS
+#define MI_USE_BLOCK_ROWS 1
+#endif
+struct BlockPlan {
+  int RT, NVT;
+  int rows() const { return (RT < 256 ? 256 : RT) / RT; }
+  int threads() const { return RT < 256 ? 256 : RT; }
+};
+inline int whole_vectors(const Common& c) { return c.V / (c.dt == MI_DTYPE_F32 ? 4 : 8); }
+inline bool block_rows_ok(const Common& c) {
+  return MI_USE_BLOCK_ROWS && 2 * (c.dt == MI_DTYPE_F32 ? 4 : 8) + c.D <= 64;
+}
+inline BlockPlan denom_block_plan(const Common& c) {
+  const int nb = whole_vectors(c);
+  if (!block_rows_ok(c) || nb <= 512) return BlockPlan{0, 0};
+  for (int nvt = 1; nvt <= 8; nvt *= 2)
+    if (nb <= 1024 * nvt) return BlockPlan{1024, nvt};
+  return BlockPlan{0, 0};
+}
+inline BlockPlan grad_block_plan(const Common& c, const void* grads) {
+  const bool same_phase = (((uintptr_t)c.acts ^ (uintptr_t)grads) & 15) == 0;
+  const int nb = whole_vectors(c);
+  if (!same_phase || !block_rows_ok(c) || nb <= 64) return BlockPlan{0, 0};
+  for (int rt = 64; rt <= 1024; rt *= 2)
+    if (nb <= 2 * rt) return BlockPlan{rt, 2};
+  for (int nvt = 4; nvt <= 8; nvt *= 2)
+    if (nb <= 1024 * nvt) return BlockPlan{1024, nvt};
+  return BlockPlan{0, 0};
+}
+inline int plan_chunks(const Common& c, const BlockPlan& p) { return (c.U + p.rows() - 1) / p.rows(); }
+inline int plan_blocks(const Common& c, const BlockPlan& p) { return plan_chunks(c, p) * c.B * c.T; }
+inline dim3 plan_grid(const Common& c, const BlockPlan& p) {
+  const unsigned turn = 8u * MI_XCD_SPAN;
+  return dim3(((unsigned)plan_blocks(c, p) + turn - 1) / turn * turn, 1, 1);
+}
+#define MI_FOR_DENOM_PLAN(P, CALL)          \
+  do {                                      \
+    if ((P).NVT == 1) CALL(1024, 1);        \
+    else if ((P).NVT == 2) CALL(1024, 2);   \
+    else if ((P).NVT == 4) CALL(1024, 4);   \
+    else CALL(1024, 8);                     \
+  } while (0)
+#define MI_FOR_GRAD_PLAN(P, CALL)           \
+  do {                                      \
+    if ((P).NVT == 8) CALL(1024, 8);        \
+    else if ((P).NVT == 4) CALL(1024, 4);   \
+    else if ((P).RT == 64) CALL(64, 2);     \
+    else if ((P).RT == 128) CALL(128, 2);   \
+    else if ((P).RT == 256) CALL(256, 2);   \
+    else if ((P).RT == 512) CALL(512, 2);   \
+    else CALL(1024, 2);                     \
+  } while (0)
+
 inline int chunks_of(const Common& c) { return (c.U + kChunkRows - 1) / kChunkRows; }
 inline int chunk_blocks(const Common& c) { return chunks_of(c) * c.B * c.T; }
 // rounded up to whole turns of the XCD permutation
@@ -1753,9 +2147,25 @@ int run_denom(const Common& c) {
                            g.bt_chunk);                                                                             \
     }                                                                                                               \
   } while (0)
-  if (c.dt == MI_DTYPE_F32) LAUNCH_DENOM(MI_DTYPE_F32);
+  const BlockPlan bp = denom_block_plan(c);
+#define LAUNCH_DENOM_BLOCK(DT, RT_, NVT_)                                                                           \
+  hipLaunchKernelGGL((denom_block_kernel<DT, RT_, NVT_>), plan_grid(c, bp), dim3(bp.threads()), 0, c.stream, c.acts, \
+                     c.labels, c.act_lens, c.label_lens, denom, arcs, c.T, c.U, c.V, c.D, c.blank, L.ND, L.Us, L.A,  \
+                     plan_chunks(c, bp), plan_blocks(c, bp))
+#define DENOM_BLOCK_F32(RT_, NVT_) LAUNCH_DENOM_BLOCK(MI_DTYPE_F32, RT_, NVT_)
+#define DENOM_BLOCK_BF16(RT_, NVT_) LAUNCH_DENOM_BLOCK(MI_DTYPE_BF16, RT_, NVT_)
+#define DENOM_BLOCK_F16(RT_, NVT_) LAUNCH_DENOM_BLOCK(MI_DTYPE_F16, RT_, NVT_)
+  if (bp.RT) {
+    if (c.dt == MI_DTYPE_F32) MI_FOR_DENOM_PLAN(bp, DENOM_BLOCK_F32);
+    else if (c.dt == MI_DTYPE_BF16) MI_FOR_DENOM_PLAN(bp, DENOM_BLOCK_BF16);
+    else MI_FOR_DENOM_PLAN(bp, DENOM_BLOCK_F16);
+  } else if (c.dt == MI_DTYPE_F32) LAUNCH_DENOM(MI_DTYPE_F32);
   else if (c.dt == MI_DTYPE_BF16) LAUNCH_DENOM(MI_DTYPE_BF16);
   else LAUNCH_DENOM(MI_DTYPE_F16);
+#undef DENOM_BLOCK_F32
+#undef DENOM_BLOCK_BF16
+#undef DENOM_BLOCK_F16
+#undef LAUNCH_DENOM_BLOCK
 #undef LAUNCH_DENOM
 #undef LAUNCH_DENOM_ROWS
   return launch_status();
@@ -1885,9 +2295,32 @@ int run_grad_stream(const Common& c, void* grads, int flags, bool fused, const S
                            c.label_lens, c.T, c.U, c.V, c.D, c.blank, L.CS, flags, g.BT, g.bt_chunk);               \
     }                                                                                                               \
   } while (0)
-  if (c.dt == MI_DTYPE_F32) LAUNCH_GRAD(MI_DTYPE_F32);
+  const BlockPlan bp = grad_block_plan(c, grads);
+#define LAUNCH_GRAD_BLOCK(DT, RT_, NVT_)                                                                            \
+  do {                                                                                                              \
+    if (fused)                                                                                                      \
+      hipLaunchKernelGGL((grad_block_kernel<DT, RT_, NVT_, true>), plan_grid(c, bp), dim3(bp.threads()), 0, c.stream, \
+                         c.acts, grads, coef, lv, c.act_lens, c.label_lens, c.T, c.U, c.V, c.D, c.blank, L.CS, flags, \
+                         plan_chunks(c, bp), plan_blocks(c, bp));                                                   \
+    else                                                                                                            \
+      hipLaunchKernelGGL((grad_block_kernel<DT, RT_, NVT_, false>), plan_grid(c, bp), dim3(bp.threads()), 0,        \
+                         c.stream, c.acts, grads, coef, lv, c.act_lens, c.label_lens, c.T, c.U, c.V, c.D, c.blank,  \
+                         L.CS, flags, plan_chunks(c, bp), plan_blocks(c, bp));                                      \
+  } while (0)
+#define GRAD_BLOCK_F32(RT_, NVT_) LAUNCH_GRAD_BLOCK(MI_DTYPE_F32, RT_, NVT_)
+#define GRAD_BLOCK_BF16(RT_, NVT_) LAUNCH_GRAD_BLOCK(MI_DTYPE_BF16, RT_, NVT_)
+#define GRAD_BLOCK_F16(RT_, NVT_) LAUNCH_GRAD_BLOCK(MI_DTYPE_F16, RT_, NVT_)
+  if (bp.RT) {
+    if (c.dt == MI_DTYPE_F32) MI_FOR_GRAD_PLAN(bp, GRAD_BLOCK_F32);
+    else if (c.dt == MI_DTYPE_BF16) MI_FOR_GRAD_PLAN(bp, GRAD_BLOCK_BF16);
+    else MI_FOR_GRAD_PLAN(bp, GRAD_BLOCK_F16);
+  } else if (c.dt == MI_DTYPE_F32) LAUNCH_GRAD(MI_DTYPE_F32);
   else if (c.dt == MI_DTYPE_BF16) LAUNCH_GRAD(MI_DTYPE_BF16);
   else LAUNCH_GRAD(MI_DTYPE_F16);
+#undef GRAD_BLOCK_F32
+#undef GRAD_BLOCK_BF16
+#undef GRAD_BLOCK_F16
+#undef LAUNCH_GRAD_BLOCK
 #undef LAUNCH_GRAD
 #undef LAUNCH_GRAD_ROWS
   return launch_status();
@@ -1957,7 +2390,7 @@ int mi_rnnt_backward(const void* acts, int act_dtype, const int64_t* labels, con
                         workspace_bytes, stream, &c);
   if (st) return st;
   const ScaleArg sc = {grad_scale, grad_scale_stride, grad_mul};
-  const bool fused = grad_rows_R(c, grads) != 0;
+  const bool fused = grad_rows_R(c, grads) != 0 || grad_block_plan(c, grads).RT != 0;
   if (!fused && (st = run_rnnt_cells(c, sc, fastemit_lambda, clamp))) return st;
   return run_grad_stream(c, grads, padding_zeroed ? kFlagPaddingDone : 0, fused, sc, fastemit_lambda, clamp);
 }
@@ -2007,7 +2440,7 @@ int mi_tdt_backward(const void* acts, int act_dtype, const int64_t* labels, cons
   if (st) return st;
   const ScaleArg sc = {grad_scale, grad_scale_stride, grad_mul};
   if (use_plain_rnnt) {  // gpu_rnnt.py:646-682: token gradient from the RNNT kernel, duration gradient stays zero
-    const bool fused = grad_rows_R(c, grads) != 0;
+    const bool fused = grad_rows_R(c, grads) != 0 || grad_block_plan(c, grads).RT != 0;
     if (!fused && (st = run_rnnt_cells(c, sc, fastemit_lambda, clamp))) return st;
     return run_grad_stream(c, grads, kFlagZeroDurations | pad_flag, fused, sc, fastemit_lambda, clamp);
   }

@@ -166,6 +166,28 @@ def test_variable_lengths_and_row_alignments(V):
         assert np.all(pad == 0)
 
 
+@pytest.mark.parametrize("V", [258, 300, 701, 1501, 3003, 5001, 9002, 20003, 33001])
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_row_lengths_of_every_kernel_family(V, dtype):
+    """Rows of 65..1024 vectors (128 to 1024 threads per row), of several vectors per thread, and rows
+    too long for either; ragged lengths so that workgroups hold live and padded rows side by side."""
+    rng = np.random.RandomState(V)
+    B, T, U = 2, 5, 5
+    acts = rng.randn(B, T, U, V) * 1.5
+    labels = rng.randint(0, V - 1, size=(B, U - 1))
+    labels[0, 0] = V - 2
+    labels[0, 1] = 0
+    act_lens, label_lens = np.array([T, 3]), np.array([2, U - 1])
+    half = dtype != torch.float32
+    costs, grads = check_against_oracle(acts, labels, act_lens, label_lens, V - 1, lam=0.001, clamp=0.3,
+                                        cost_rtol=1e-6, grad_atol=2.0**-8 if half else 2e-6,
+                                        dtype=dtype)  # fmt: skip
+    for b in range(B):
+        pad = grads[b].copy()
+        pad[: act_lens[b], : label_lens[b] + 1] = 0
+        assert np.all(pad == 0)
+
+
 @pytest.mark.parametrize("U", [1, 2, 64, 65, 129, 257])
 def test_label_axis_sizes(U):
     """U = 1 (empty transcripts), wave boundaries (64/65) and the 2, 4 and 8 cells-per-lane kernels."""

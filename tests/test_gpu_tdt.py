@@ -46,7 +46,7 @@ def test_random_cases_like_the_reference(durations):
     check_against_oracle(acts, labels, [T] * B, [U - 1] * B, V, durations, 0.05)
 
 
-@pytest.mark.parametrize("V", [4, 29, 1025])
+@pytest.mark.parametrize("V", [4, 29, 301, 1025, 2500, 5001])
 def test_variable_lengths_fastemit_clamp(V):
     rng = np.random.RandomState(V + 1)
     durations = [0, 1, 2, 3, 4]
