@@ -228,6 +228,32 @@ template <bool NT> __device__ __forceinline__ uint4 load_stream(const uint4* p) 
   }
 }
 
+// n / d for n < 2^31 by one multiply and one shift (the round-up multiplier of Granlund and
+// Montgomery, "Division by invariant integers using multiplication"): the hardware has no integer
+// divide, and the two divisions that split a workgroup id into (b, t, chunk) would otherwise cost
+// some sixty instructions at the head of every wave.
+struct FastDiv {
+  unsigned mul, shift;
+};
+inline FastDiv make_fastdiv(unsigned d) {
+  unsigned l = 0;
+  while ((1ull << l) < d) ++l;
+  FastDiv f;
+  f.mul = (unsigned)((((unsigned long long)1 << 32) * (((unsigned long long)1 << l) - d)) / d + 1);
+  f.shift = l;
+  return f;
+}
+__device__ __forceinline__ unsigned fast_div(unsigned n, FastDiv f) { return (__umulhi(n, f.mul) + n) >> f.shift; }
+struct GridDiv {
+  FastDiv chunks, T;
+};
+inline GridDiv make_griddiv(int nchunks, int T) {
+  GridDiv g;
+  g.chunks = make_fastdiv((unsigned)nchunks);
+  g.T = make_fastdiv((unsigned)T);
+  return g;
+}
+
 // Workgroups are dealt round-robin to the 8 XCDs in launch order.  The logical block id is
 // permuted so that each XCD takes MI_XCD_SPAN consecutive logical blocks (a contiguous piece
 // of the tensor) per turn: contiguous enough for the XCD's own L2 and TLB to see a linear
@@ -338,9 +364,10 @@ struct UttLens {
 __device__ __forceinline__ UttLens load_lens(const int64_t* act_lens, const int64_t* label_lens, int b, int T, int U) {
   long long len_t = uni((long long)sload(act_lens + b)), len_u = uni((long long)sload(label_lens + b));
   asm("" : "+s"(len_t), "+s"(len_u));
+  // a length outside [0, limit] (never seen from a checked caller) is taken as the limit
   UttLens r;
-  r.Tb = clampi(len_t, 1, T);
-  r.Ub = clampi(len_u + 1, 1, U);
+  r.Tb = max((unsigned long long)len_t > (unsigned)T ? T : (int)len_t, 1);
+  r.Ub = max((unsigned long long)len_u >= (unsigned)U ? U : (int)len_u + 1, 1);
   return r;
 }
 
@@ -1373,13 +1400,14 @@ template <int DT, int R>
 __global__ __launch_bounds__(kRowThreads) void denom_rows_kernel(
     const void* __restrict__ acts, const int64_t* __restrict__ labels, const int64_t* __restrict__ act_lens,
     const int64_t* __restrict__ label_lens, float* __restrict__ denom, float* __restrict__ arcs, int T, int U, int V,
-    int D, int blank, int ND, int Us, int A, int nchunks, int nblocks) {
+    int D, int blank, int ND, int Us, int A, int nchunks, int nblocks, GridDiv gdiv) {
   constexpr int VEC = Elem<DT>::VEC;
   // all kernel arguments are fetched in one go, not one batch per use (the loads this kernel wants
   // on the scalar unit are written as such, so the asm's side effect costs nothing)
   asm volatile("" ::"s"((uintptr_t)acts), "s"((uintptr_t)labels), "s"((uintptr_t)act_lens), "s"((uintptr_t)label_lens),
                "s"((uintptr_t)denom), "s"((uintptr_t)arcs), "s"(T), "s"(U), "s"(V), "s"(D), "s"(blank), "s"(ND), "s"(Us),
-               "s"(A), "s"(nchunks), "s"(nblocks));
+               "s"(A), "s"(nchunks), "s"(nblocks), "s"(gdiv.chunks.mul), "s"(gdiv.chunks.shift), "s"(gdiv.T.mul),
+               "s"(gdiv.T.shift));
   const int lane = threadIdx.x & 63;
   const int wave = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
   // 1-D grid over (b,t,chunk), chunk fastest = memory order
@@ -1388,8 +1416,8 @@ __global__ __launch_bounds__(kRowThreads) void denom_rows_kernel(
 #if MI_K1_REVERSE
   wg = (unsigned)nblocks - 1u - wg;
 #endif
-  const unsigned bt = wg / (unsigned)nchunks, chunk = wg - bt * (unsigned)nchunks;
-  const int b = (int)(bt / (unsigned)T), t = (int)(bt - (unsigned)b * (unsigned)T);
+  const unsigned bt = fast_div(wg, gdiv.chunks), chunk = wg - bt * (unsigned)nchunks;
+  const int b = (int)fast_div(bt, gdiv.T), t = (int)(bt - (unsigned)b * (unsigned)T);
   const int u_begin = (int)chunk * kChunkRows + wave;
   // the wave's label ids travel with the lengths (a clamped index, dropped below if the row has no
   // label arc; with U == 1 there is no label array and a length is read instead)
@@ -1407,7 +1435,7 @@ __global__ __launch_bounds__(kRowThreads) void denom_rows_kernel(
   const int u_end = min(Ub, (int)(chunk + 1) * kChunkRows);
   if (u_begin >= u_end) return;
   const int VD = V + D;
-  const size_t cell0 = ((size_t)b * T + t) * U;
+  const unsigned cell0 = ((unsigned)b * (unsigned)T + (unsigned)t) * (unsigned)U;  // B*T*U < 2^31 (host check)
 
   // the wave's label ids, fetched once so that no row waits on an id before asking for its logit
   int labs[kRowsPerWave];
@@ -1423,7 +1451,7 @@ __global__ __launch_bounds__(kRowThreads) void denom_rows_kernel(
     int mis;
   };
   auto fetch = [&](int uu, int lab, Row& d) {
-    const size_t e0 = (cell0 + uu) * VD;
+    const size_t e0 = (size_t)(cell0 + (unsigned)uu) * (unsigned)VD;
     const RowWindow<DT> w(acts, e0);
     const RowSplit<DT> sp(w.mis, V);
     d.mis = w.mis;
@@ -1506,7 +1534,7 @@ __global__ __launch_bounds__(kRowThreads) void grad_rows_kernel(const void* __re
                                                         const int64_t* __restrict__ act_lens,
                                                         const int64_t* __restrict__ label_lens, int T, int U, int V,
                                                         int D, int blank, int CS, int flags, int nchunks,
-                                                        int nblocks) {
+                                                        int nblocks, GridDiv gdiv) {
   constexpr int VEC = Elem<DT>::VEC;
   // all kernel arguments are fetched in one go, not one batch per use (the loads this kernel wants
   // on the scalar unit are written as such, so the asm's side effect costs nothing)
@@ -1515,7 +1543,7 @@ __global__ __launch_bounds__(kRowThreads) void grad_rows_kernel(const void* __re
                "s"((uintptr_t)lv.betas), "s"((uintptr_t)lv.ll), "s"((uintptr_t)lv.labels), "s"((uintptr_t)lv.grad_scale),
                "s"(lv.grad_scale_stride), "s"(lv.grad_mul), "s"(lv.ND), "s"(lv.Us), "s"(lv.A), "s"(lv.lambda),
                "s"(lv.clamp), "s"(T), "s"(U), "s"(V), "s"(D), "s"(blank), "s"(CS), "s"(flags), "s"(nchunks),
-               "s"(nblocks));
+               "s"(nblocks), "s"(gdiv.chunks.mul), "s"(gdiv.chunks.shift), "s"(gdiv.T.mul), "s"(gdiv.T.shift));
   const int lane = threadIdx.x & 63;
   const int wave = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
   // 1-D grid over (b,t,chunk), chunk fastest = memory order
@@ -1524,17 +1552,17 @@ __global__ __launch_bounds__(kRowThreads) void grad_rows_kernel(const void* __re
 #if MI_K4_REVERSE
   wg = (unsigned)nblocks - 1u - wg;
 #endif
-  const unsigned bt = wg / (unsigned)nchunks, chunk = wg - bt * (unsigned)nchunks;
-  const int b = (int)(bt / (unsigned)T), t = (int)(bt - (unsigned)b * (unsigned)T);
+  const unsigned bt = fast_div(wg, gdiv.chunks), chunk = wg - bt * (unsigned)nchunks;
+  const int b = (int)fast_div(bt, gdiv.T), t = (int)(bt - (unsigned)b * (unsigned)T);
   const UttLens len = load_lens(act_lens, label_lens, b, T, U);
   const int Tb = len.Tb, Ub = len.Ub;
   const int VD = V + D;
-  const size_t cell0 = ((size_t)b * T + t) * U;
+  const unsigned cell0 = ((unsigned)b * (unsigned)T + (unsigned)t) * (unsigned)U;  // B*T*U < 2^31 (host check)
   const int c0 = (int)chunk * kChunkRows;
   const int c1 = min(U, c0 + kChunkRows);
   // rows [c0, z0) of this chunk carry a gradient, rows [z0, c1) are padding: one contiguous range of zeros
   const int z0 = (t >= Tb) ? c0 : max(c0, min(Ub, c1));
-  if (!(flags & kFlagPaddingDone)) zero_elems<DT>(grads, (cell0 + z0) * VD, (cell0 + c1) * VD);
+  if (!(flags & kFlagPaddingDone)) zero_elems<DT>(grads, (size_t)(cell0 + z0) * VD, (size_t)(cell0 + c1) * VD);
   const int u_begin = c0 + wave;
   if (u_begin >= z0) return;
 
@@ -1551,7 +1579,7 @@ __global__ __launch_bounds__(kRowThreads) void grad_rows_kernel(const void* __re
     return v;
   };
   auto fetch = [&](int uu, Row& d) {
-    const size_t e0 = (cell0 + uu) * VD;
+    const size_t e0 = (size_t)(cell0 + (unsigned)uu) * (unsigned)VD;
     const RowWindow<DT> w(acts, e0);
     const RowSplit<DT> sp(w.mis, V);
     d.mis = w.mis;
@@ -1565,7 +1593,7 @@ __global__ __launch_bounds__(kRowThreads) void grad_rows_kernel(const void* __re
       d.c = finish_coef(cr, lv, t, uu, Tb, Ub, V, blank);
       d.gd = 0.f;
     } else {
-      const float* c = coef + (cell0 + uu) * CS;
+      const float* c = coef + (size_t)(cell0 + uu) * CS;
       const float4 ca = *(const float4*)c;        // denom*log2e, W*scale, clamp bound, G_blank
       const float2 cb = *(const float2*)(c + 4);  // G_label, label id
       d.c.dl2 = ca.x; d.c.W = ca.y; d.c.cb = ca.z; d.c.gB = ca.w; d.c.gL = cb.x;
@@ -1574,7 +1602,7 @@ __global__ __launch_bounds__(kRowThreads) void grad_rows_kernel(const void* __re
     }
   };
   auto emit = [&](int uu, const Row& d) {
-    const size_t e0 = (cell0 + uu) * VD;
+    const size_t e0 = (size_t)(cell0 + (unsigned)uu) * (unsigned)VD;
     const RowSplit<DT> sp(d.mis, V);
     const float dl2 = d.c.dl2, W = d.c.W, cb = d.c.cb, gB = d.c.gB, gL = d.c.gL;
     const int lab = d.c.lab;
@@ -1637,18 +1665,18 @@ template <int DT>
 __global__ __launch_bounds__(kRowThreads) void zero_padding_kernel(void* __restrict__ grads,
                                                                    const int64_t* __restrict__ act_lens,
                                                                    const int64_t* __restrict__ label_lens, int T,
-                                                                   int U, int VD, int nchunks, int nblocks) {
+                                                                   int U, int VD, int nchunks, int nblocks, GridDiv gdiv) {
   const unsigned wg = logical_block();
   if (wg >= (unsigned)nblocks) return;
-  const unsigned bt = wg / (unsigned)nchunks, chunk = wg - bt * (unsigned)nchunks;
-  const int b = (int)(bt / (unsigned)T), t = (int)(bt - (unsigned)b * (unsigned)T);
+  const unsigned bt = fast_div(wg, gdiv.chunks), chunk = wg - bt * (unsigned)nchunks;
+  const int b = (int)fast_div(bt, gdiv.T), t = (int)(bt - (unsigned)b * (unsigned)T);
   const int Tb = clampi(act_lens[b], 1, T);
   const int Ub = clampi(label_lens[b] + 1, 1, U);
-  const size_t cell0 = ((size_t)b * T + t) * U;
+  const unsigned cell0 = ((unsigned)b * (unsigned)T + (unsigned)t) * (unsigned)U;  // B*T*U < 2^31 (host check)
   const int c0 = (int)chunk * kChunkRows;
   const int c1 = min(U, c0 + kChunkRows);
   const int z0 = (t >= Tb) ? c0 : max(c0, min(Ub, c1));
-  zero_elems<DT>(grads, (cell0 + z0) * VD, (cell0 + c1) * VD);
+  zero_elems<DT>(grads, (size_t)(cell0 + z0) * VD, (size_t)(cell0 + c1) * VD);
 }
 
 // ----------------------------------------------------------------------------------------
@@ -1667,7 +1695,7 @@ template <int DT, int RT, int NVT>
 __global__ __launch_bounds__(BlockRows<RT>::THREADS) void denom_block_kernel(
     const void* __restrict__ acts, const int64_t* __restrict__ labels, const int64_t* __restrict__ act_lens,
     const int64_t* __restrict__ label_lens, float* __restrict__ denom, float* __restrict__ arcs, int T, int U, int V,
-    int D, int blank, int ND, int Us, int A, int nchunks, int nblocks) {
+    int D, int blank, int ND, int Us, int A, int nchunks, int nblocks, GridDiv gdiv) {
   constexpr int VEC = Elem<DT>::VEC;
   constexpr int ROWS = BlockRows<RT>::ROWS, WPR = BlockRows<RT>::WPR, WAVES = BlockRows<RT>::THREADS / 64;
   __shared__ float2 part[WAVES];
@@ -1675,7 +1703,8 @@ __global__ __launch_bounds__(BlockRows<RT>::THREADS) void denom_block_kernel(
   // on the scalar unit are written as such, so the asm's side effect costs nothing)
   asm volatile("" ::"s"((uintptr_t)acts), "s"((uintptr_t)labels), "s"((uintptr_t)act_lens), "s"((uintptr_t)label_lens),
                "s"((uintptr_t)denom), "s"((uintptr_t)arcs), "s"(T), "s"(U), "s"(V), "s"(D), "s"(blank), "s"(ND), "s"(Us),
-               "s"(A), "s"(nchunks), "s"(nblocks));
+               "s"(A), "s"(nchunks), "s"(nblocks), "s"(gdiv.chunks.mul), "s"(gdiv.chunks.shift), "s"(gdiv.T.mul),
+               "s"(gdiv.T.shift));
   const int lane = threadIdx.x & 63;
   const int wave = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
   const int row_in_wg = wave / WPR, wave_in_row = wave - row_in_wg * WPR;
@@ -1685,8 +1714,8 @@ __global__ __launch_bounds__(BlockRows<RT>::THREADS) void denom_block_kernel(
 #if MI_K1_REVERSE
   wg = (unsigned)nblocks - 1u - wg;
 #endif
-  const unsigned bt = wg / (unsigned)nchunks, chunk = wg - bt * (unsigned)nchunks;
-  const int b = (int)(bt / (unsigned)T), t = (int)(bt - (unsigned)b * (unsigned)T);
+  const unsigned bt = fast_div(wg, gdiv.chunks), chunk = wg - bt * (unsigned)nchunks;
+  const int b = (int)fast_div(bt, gdiv.T), t = (int)(bt - (unsigned)b * (unsigned)T);
   const int u = (int)chunk * ROWS + row_in_wg;
   // the row's label id travels with the lengths (a clamped index, dropped below if the row has no
   // label arc; with U == 1 there is no label array and a length is read instead)
@@ -1697,8 +1726,8 @@ __global__ __launch_bounds__(BlockRows<RT>::THREADS) void denom_block_kernel(
   if (t >= Tb || (int)chunk * ROWS >= Ub) return;  // the whole workgroup leaves: no barrier is left waiting
   const bool live = u < Ub;  // wave-uniform
   const int VD = V + D;
-  const size_t cell0 = ((size_t)b * T + t) * U;
-  const size_t e0 = (cell0 + (live ? u : 0)) * VD;
+  const unsigned cell0 = ((unsigned)b * (unsigned)T + (unsigned)t) * (unsigned)U;  // B*T*U < 2^31 (host check)
+  const size_t e0 = (size_t)(cell0 + (unsigned)(live ? u : 0)) * (unsigned)VD;
 
   float m_w = -1.0e30f, s_w = 0.f;  // this wave's share of the row: max and sum of 2^((x - max) log2 e)
   float xb = 0.f, xl = 0.f, xd = 0.f;
@@ -1773,7 +1802,7 @@ template <int DT, int RT, int NVT, bool FUSED>
 __global__ __launch_bounds__(BlockRows<RT>::THREADS) void grad_block_kernel(
     const void* __restrict__ acts, void* __restrict__ grads, const float* __restrict__ coef, LatticeView lv,
     const int64_t* __restrict__ act_lens, const int64_t* __restrict__ label_lens, int T, int U, int V, int D,
-    int blank, int CS, int flags, int nchunks, int nblocks) {
+    int blank, int CS, int flags, int nchunks, int nblocks, GridDiv gdiv) {
   constexpr int VEC = Elem<DT>::VEC;
   constexpr int ROWS = BlockRows<RT>::ROWS, WPR = BlockRows<RT>::WPR;
   // all kernel arguments are fetched in one go, not one batch per use (the loads this kernel wants
@@ -1783,7 +1812,7 @@ __global__ __launch_bounds__(BlockRows<RT>::THREADS) void grad_block_kernel(
                "s"((uintptr_t)lv.betas), "s"((uintptr_t)lv.ll), "s"((uintptr_t)lv.labels), "s"((uintptr_t)lv.grad_scale),
                "s"(lv.grad_scale_stride), "s"(lv.grad_mul), "s"(lv.ND), "s"(lv.Us), "s"(lv.A), "s"(lv.lambda),
                "s"(lv.clamp), "s"(T), "s"(U), "s"(V), "s"(D), "s"(blank), "s"(CS), "s"(flags), "s"(nchunks),
-               "s"(nblocks));
+               "s"(nblocks), "s"(gdiv.chunks.mul), "s"(gdiv.chunks.shift), "s"(gdiv.T.mul), "s"(gdiv.T.shift));
   const int lane = threadIdx.x & 63;
   const int wave = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
   const int row_in_wg = wave / WPR, wave_in_row = wave - row_in_wg * WPR;
@@ -1793,15 +1822,15 @@ __global__ __launch_bounds__(BlockRows<RT>::THREADS) void grad_block_kernel(
 #if MI_K4_REVERSE
   wg = (unsigned)nblocks - 1u - wg;
 #endif
-  const unsigned bt = wg / (unsigned)nchunks, chunk = wg - bt * (unsigned)nchunks;
-  const int b = (int)(bt / (unsigned)T), t = (int)(bt - (unsigned)b * (unsigned)T);
+  const unsigned bt = fast_div(wg, gdiv.chunks), chunk = wg - bt * (unsigned)nchunks;
+  const int b = (int)fast_div(bt, gdiv.T), t = (int)(bt - (unsigned)b * (unsigned)T);
   const int u = (int)chunk * ROWS + row_in_wg;
   if (u >= U) return;
   const UttLens len = load_lens(act_lens, label_lens, b, T, U);
   const int Tb = len.Tb, Ub = len.Ub;
   const int VD = V + D;
-  const size_t cell0 = ((size_t)b * T + t) * U;
-  const size_t e0 = (cell0 + u) * VD;
+  const unsigned cell0 = ((unsigned)b * (unsigned)T + (unsigned)t) * (unsigned)U;  // B*T*U < 2^31 (host check)
+  const size_t e0 = (size_t)(cell0 + (unsigned)u) * (unsigned)VD;
   const RowWindow<DT> w(acts, e0);
   const RowSplit<DT> sp(w.mis, V);
   char* grow = (char*)grads + e0 * Elem<DT>::BYTES;  // same 16-byte phase as the acts row
@@ -1833,7 +1862,7 @@ __global__ __launch_bounds__(BlockRows<RT>::THREADS) void grad_block_kernel(
     const CoefRaw cr = load_coef_raw(lv, b, t, u, Tb, Ub, T, U);
     c = finish_coef(cr, lv, t, u, Tb, Ub, V, blank);
   } else {
-    const float* cp = coef + (cell0 + u) * CS;
+    const float* cp = coef + (size_t)(cell0 + u) * CS;
     const float4 ca = *(const float4*)cp;        // denom*log2e, W*scale, clamp bound, G_blank
     const float2 cb = *(const float2*)(cp + 4);  // G_label, label id
     c.dl2 = ca.x; c.W = ca.y; c.cb = ca.z; c.gB = ca.w; c.gL = cb.x;
@@ -2133,7 +2162,7 @@ int run_denom(const Common& c) {
   ProfScope prof(MI_PROFILE_DENOM, c.stream);
 #define LAUNCH_DENOM_ROWS(DT, RR)                                                                                   \
   hipLaunchKernelGGL((denom_rows_kernel<DT, RR>), chunk_grid(c), dim3(kRowThreads), 0, c.stream, c.acts, c.labels,           \
-                     c.act_lens, c.label_lens, denom, arcs, c.T, c.U, c.V, c.D, c.blank, L.ND, L.Us, L.A, chunks_of(c), chunk_blocks(c))
+                     c.act_lens, c.label_lens, denom, arcs, c.T, c.U, c.V, c.D, c.blank, L.ND, L.Us, L.A, chunks_of(c), chunk_blocks(c), make_griddiv(chunks_of(c), c.T))
 #define LAUNCH_DENOM(DT)                                                                                            \
   do {                                                                                                              \
     switch (R) {                                                                                                    \
@@ -2151,7 +2180,7 @@ int run_denom(const Common& c) {
 #define LAUNCH_DENOM_BLOCK(DT, RT_, NVT_)                                                                           \
   hipLaunchKernelGGL((denom_block_kernel<DT, RT_, NVT_>), plan_grid(c, bp), dim3(bp.threads()), 0, c.stream, c.acts, \
                      c.labels, c.act_lens, c.label_lens, denom, arcs, c.T, c.U, c.V, c.D, c.blank, L.ND, L.Us, L.A,  \
-                     plan_chunks(c, bp), plan_blocks(c, bp))
+                     plan_chunks(c, bp), plan_blocks(c, bp), make_griddiv(plan_chunks(c, bp), c.T))
 #define DENOM_BLOCK_F32(RT_, NVT_) LAUNCH_DENOM_BLOCK(MI_DTYPE_F32, RT_, NVT_)
 #define DENOM_BLOCK_BF16(RT_, NVT_) LAUNCH_DENOM_BLOCK(MI_DTYPE_BF16, RT_, NVT_)
 #define DENOM_BLOCK_F16(RT_, NVT_) LAUNCH_DENOM_BLOCK(MI_DTYPE_F16, RT_, NVT_)
@@ -2277,11 +2306,11 @@ int run_grad_stream(const Common& c, void* grads, int flags, bool fused, const S
     if (fused)                                                                                                      \
       hipLaunchKernelGGL((grad_rows_kernel<DT, RR, true>), chunk_grid(c), dim3(kRowThreads), 0, c.stream, c.acts, grads,     \
                          coef, lv, c.act_lens, c.label_lens, c.T, c.U, c.V, c.D, c.blank, L.CS, flags,               \
-                         chunks_of(c), chunk_blocks(c));                                                            \
+                         chunks_of(c), chunk_blocks(c), make_griddiv(chunks_of(c), c.T));                                                            \
     else                                                                                                            \
       hipLaunchKernelGGL((grad_rows_kernel<DT, RR, false>), chunk_grid(c), dim3(kRowThreads), 0, c.stream, c.acts, grads,    \
                          coef, lv, c.act_lens, c.label_lens, c.T, c.U, c.V, c.D, c.blank, L.CS, flags,               \
-                         chunks_of(c), chunk_blocks(c));                                                            \
+                         chunks_of(c), chunk_blocks(c), make_griddiv(chunks_of(c), c.T));                                                            \
   } while (0)
 #define LAUNCH_GRAD(DT)                                                                                             \
   do {                                                                                                              \
@@ -2301,11 +2330,11 @@ int run_grad_stream(const Common& c, void* grads, int flags, bool fused, const S
     if (fused)                                                                                                      \
       hipLaunchKernelGGL((grad_block_kernel<DT, RT_, NVT_, true>), plan_grid(c, bp), dim3(bp.threads()), 0, c.stream, \
                          c.acts, grads, coef, lv, c.act_lens, c.label_lens, c.T, c.U, c.V, c.D, c.blank, L.CS, flags, \
-                         plan_chunks(c, bp), plan_blocks(c, bp));                                                   \
+                         plan_chunks(c, bp), plan_blocks(c, bp), make_griddiv(plan_chunks(c, bp), c.T));                                                   \
     else                                                                                                            \
       hipLaunchKernelGGL((grad_block_kernel<DT, RT_, NVT_, false>), plan_grid(c, bp), dim3(bp.threads()), 0,        \
                          c.stream, c.acts, grads, coef, lv, c.act_lens, c.label_lens, c.T, c.U, c.V, c.D, c.blank,  \
-                         L.CS, flags, plan_chunks(c, bp), plan_blocks(c, bp));                                      \
+                         L.CS, flags, plan_chunks(c, bp), plan_blocks(c, bp), make_griddiv(plan_chunks(c, bp), c.T));                                      \
   } while (0)
 #define GRAD_BLOCK_F32(RT_, NVT_) LAUNCH_GRAD_BLOCK(MI_DTYPE_F32, RT_, NVT_)
 #define GRAD_BLOCK_BF16(RT_, NVT_) LAUNCH_GRAD_BLOCK(MI_DTYPE_BF16, RT_, NVT_)
@@ -2535,7 +2564,7 @@ int mi_transducer_zero_padding(void* grads, int act_dtype, const int64_t* act_le
   ProfScope prof(MI_PROFILE_ZERO, (hipStream_t)stream);
 #define LAUNCH_ZERO(DT)                                                                                          \
   hipLaunchKernelGGL(zero_padding_kernel<DT>, grid, dim3(kRowThreads), 0, (hipStream_t)stream, grads, act_lens,   \
-                     label_lens, T, U, VD, nchunks, nblocks)
+                     label_lens, T, U, VD, nchunks, nblocks, make_griddiv(nchunks, T))
   if (act_dtype == MI_DTYPE_F32) LAUNCH_ZERO(MI_DTYPE_F32);
   else if (act_dtype == MI_DTYPE_BF16) LAUNCH_ZERO(MI_DTYPE_BF16);
   else LAUNCH_ZERO(MI_DTYPE_F16);
