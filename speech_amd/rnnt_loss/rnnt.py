@@ -67,10 +67,15 @@ def new_workspace(acts, num_durations=0):
     return torch.empty(nbytes, dtype=torch.uint8, device=acts.device)
 
 
-def length_maxima(act_lens, label_lens):
-    """Device int64[2] = (max(act_lens), max(label_lens)), enqueued on the current stream."""
+def length_maxima(act_lens, label_lens, out=None):
+    """int64[2] = (max(act_lens), max(label_lens)), enqueued on the current stream.  `out` may be a
+    pinned host tensor: the kernel then writes the two values straight into host memory (pinned
+    allocations are mapped into the device's address space), which saves the copy back."""
     _require_gpu(act_lens, "length_maxima")
-    out = torch.empty(2, dtype=torch.int64, device=act_lens.device)
+    if out is None:
+        out = torch.empty(2, dtype=torch.int64, device=act_lens.device)
+    elif out.dtype != torch.int64 or out.numel() != 2 or not (out.is_cuda or out.is_pinned()):
+        raise ValueError("length_maxima: out must be an int64[2] device or pinned host tensor")
     with torch.cuda.device(act_lens.device):
         status = _native.lib().mi_transducer_length_maxima(
             _ptr(act_lens), _ptr(label_lens), act_lens.shape[0], _ptr(out), _stream(act_lens.device)

@@ -87,11 +87,19 @@ class _PendingLengthCheck:
     def __init__(self, log_probs, lengths, label_lengths):
         self.T, self.U = log_probs.shape[1:3]
         if lengths.is_cuda:
-            maxima = rnnt.length_maxima(lengths, label_lengths)
+            # One small kernel on the auxiliary stream, ordered after whatever produced the lengths
+            # on the current stream, writes the two maxima into pinned host memory: it runs beside
+            # the first kernel of the loss instead of in front of it.
+            main = torch.cuda.current_stream(lengths.device)
+            aux = _aux_stream(lengths.device)
+            aux.wait_stream(main)
             self.host = torch.empty(2, dtype=torch.int64, pin_memory=True)
-            self.host.copy_(maxima, non_blocking=True)
-            self.event = torch.cuda.Event()
-            self.event.record(torch.cuda.current_stream(lengths.device))
+            with torch.cuda.stream(aux):
+                rnnt.length_maxima(lengths, label_lengths, out=self.host)
+                self.event = torch.cuda.Event()
+                self.event.record(aux)
+            lengths.record_stream(aux)
+            label_lengths.record_stream(aux)
         else:
             self.host = torch.stack([torch.max(lengths), torch.max(label_lengths)])
             self.event = None
