@@ -549,7 +549,8 @@ template <int K> __device__ __forceinline__ void store_k(double* p, const double
 
 // Arc log-probs of cells outside the utterance's lattice were never written: whatever bits
 // are there must not turn a -inf lattice value into NaN, so they are forced finite.
-__device__ __forceinline__ float finite_arc(float x) { return fminf(fmaxf(x, -3.0e38f), 3.0e38f); }
+// (one median-of-three instruction; a NaN comes out as the lower bound)
+__device__ __forceinline__ float finite_arc(float x) { return __builtin_amdgcn_fmed3f(x, -3.0e38f, 3.0e38f); }
 
 // RNNT lattice: one wave per (utterance, direction).  Lane l owns columns u = l*K .. l*K+K-1
 // and, at step n, the cells (n-u, u) of anti-diagonal n.

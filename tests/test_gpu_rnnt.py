@@ -188,7 +188,7 @@ def test_row_lengths_of_every_kernel_family(V, dtype):
         assert np.all(pad == 0)
 
 
-@pytest.mark.parametrize("U", [1, 2, 64, 65, 129, 257])
+@pytest.mark.parametrize("U", [1, 2, 64, 65, 129, 257, 600])
 def test_label_axis_sizes(U):
     """U = 1 (empty transcripts), wave boundaries (64/65) and the 2, 4 and 8 cells-per-lane kernels."""
     rng = np.random.RandomState(U)
