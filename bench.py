@@ -6,8 +6,9 @@ A step is one forward + backward of the loss module over one resident batch:
 on the north-star workload (RNNT, B=16, T=375, U+1=121, V=1025, fp32, variable
 lengths), inputs already in HBM.  Prints ONE JSON line:
   value        logit elements per second (B*T*U*V / step time)
-  roofline     the gradient-stream kernel (the dominant one): algorithmic bytes per launch /
-               its mean duration, measured with HIP events around the launches of the timed steps
+  roofline     the gradient pass (the dominant kernel; its name for this shape is reported):
+               algorithmic bytes per launch / its mean duration, measured with HIP events around
+               the launches of the timed steps
   cpu_baseline the C restatement of the reference's CPU path on a bounded sample, host cores
   kernels      mean duration of each pipeline kernel over the timed steps (ms)
   copy_probe   bandwidth a plain device copy reaches on this GPU (GB/s, read + write)
@@ -28,7 +29,7 @@ if ROOT not in sys.path:
 
 HBM_PEAK_GBPS = 8000.0  # MI355X HBM3E, published peak
 
-# HBM bytes per launch of grad_stream_kernel from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of
+# HBM bytes per launch of the gradient-pass kernel from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of
 # this script, scaled by what the same counters read for mi_transducer_copy_probe of known size
 # (summaries under profiles/).  None = not measured for that workload.
 MEASURED_TRAFFIC_BYTES = {
@@ -117,7 +118,7 @@ def main():
 
     # the timed region: only the dominant kernel is bracketed by events (an event pair costs
     # a few microseconds of queue time; the other kernels are timed in a separate pass below)
-    _native.profile_enable(args.steps, ["grad_stream_kernel"])
+    _native.profile_enable(args.steps, ["gradient_pass"])
     start_ev, stop_ev = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
     torch.cuda.synchronize()
     t0 = time.perf_counter()
@@ -155,9 +156,12 @@ def main():
     copy_gbps = 2 * n * 10 / (e0.elapsed_time(e1) * 1e-3) / 1e9
     del src, dst
 
-    from speech_amd.rnnt_loss import rnnt_pytorch
+    from speech_amd.rnnt_loss import rnnt, rnnt_pytorch
 
-    grad_ms, grad_n = kernels["grad_stream_kernel"]
+    plan = _native.describe_plan(rnnt._dtype_code(acts), cfg.B, cfg.T, cfg.U, cfg.V, cfg.D,
+                                 max(cfg.durations) if cfg.D else 0)  # fmt: skip
+
+    grad_ms, grad_n = kernels["gradient_pass"]
     grad_avg_s = grad_ms * 1e-3 / max(grad_n, 1)
     # with the padding zero-filled by its own kernel during forward, the gradient pass reads and
     # writes the valid rows only
@@ -190,7 +194,7 @@ def main():
             "event_ms_per_step": event_ms_per_step,
         },
         "roofline": {
-            "kernel": "grad_stream_kernel",
+            "kernel": plan["gradient"],
             "bound": "hbm",
             "achieved": achieved,
             "peak": HBM_PEAK_GBPS,
@@ -203,6 +207,7 @@ def main():
             "launches": grad_n,
         },
         "kernels": {k: (ms / max(n_, 1)) for k, (ms, n_) in breakdown.items()},
+        "plan": plan,
         "copy_probe_GBps": copy_gbps,
     }  # fmt: skip
     if not args.no_cpu_baseline:

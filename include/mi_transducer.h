@@ -167,15 +167,23 @@ int mi_transducer_length_maxima(const int64_t* act_lens, const int64_t* label_le
  * select only the kernel it needs.  mi_transducer_profile_read waits for the recorded
  * launches of one kernel class, returns their summed duration and count, and resets that
  * class.  Not thread-safe; leave disabled outside benchmarks. */
-#define MI_PROFILE_DENOM 0   /* denom_rows_kernel / denom_gather_kernel */
-#define MI_PROFILE_LATTICE 1 /* rnnt_lattice_kernel / tdt_lattice_kernel */
+#define MI_PROFILE_DENOM 0   /* denom_rows_kernel / denom_block_kernel / denom_gather_kernel */
+#define MI_PROFILE_LATTICE 1 /* rnnt_lattice_kernel / tdt_lattice_block_kernel / tdt_lattice_kernel */
 #define MI_PROFILE_CELL 2    /* rnnt_cell_kernel / tdt_cell_kernel */
-#define MI_PROFILE_GRAD 3    /* grad_rows_kernel / grad_stream_kernel */
+#define MI_PROFILE_GRAD 3    /* grad_rows_kernel / grad_block_kernel / grad_stream_kernel */
 #define MI_PROFILE_ZERO 4    /* zero_padding_kernel */
 #define MI_PROFILE_KERNELS 5
 int mi_transducer_profile_enable(int max_launches, unsigned kernel_mask);
 int mi_transducer_profile_read(int kernel_id, float* total_ms, int* launches);
 int mi_transducer_profile_disable(void);
+
+/* Which kernels a call with this shape would launch, as text:
+ * "denominators=...; lattice=...; cells=...; gradient=..." ("cells=-" when the gradient pass derives
+ * its coefficients itself).  D = 0 for RNNT; for TDT pass the largest duration.  Assumes a gradient
+ * buffer at the 16-byte phase of the logits.  Launches nothing.  For benchmarks, profiles and tests
+ * that want to name (or pin) the kernel family a shape maps to. */
+int mi_transducer_describe_plan(int act_dtype, int B, int T, int U, int V, int D, int max_duration,
+                                int use_plain_rnnt, char* out, size_t out_bytes);
 
 /* Plain device-to-device copy of `bytes` (multiple of 16, 16-byte aligned pointers) with a
  * grid-stride 16-byte-per-lane kernel: the known-size yardstick for hardware traffic

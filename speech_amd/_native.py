@@ -16,7 +16,7 @@ INCLUDE_DIR = os.path.join(os.path.dirname(_HERE), "include")
 LIB_PATH = os.environ.get("MI_TRANSDUCER_LIB") or os.path.join(CSRC_DIR, "libmi_transducer.so")
 SOURCES = [os.path.join(CSRC_DIR, "mi_transducer.hip")]
 
-ABI_VERSION = 5
+ABI_VERSION = 6
 SUCCESS, INVALID_VALUE, LAUNCH_FAILURE = 0, 1, 2
 DTYPE_F32, DTYPE_BF16, DTYPE_F16 = 0, 1, 2
 
@@ -79,6 +79,8 @@ _SIGNATURES = {
     "mi_transducer_profile_enable": [_c_int, ctypes.c_uint],
     "mi_transducer_profile_read": [_c_int, ctypes.POINTER(_c_float), ctypes.POINTER(_c_int)],
     "mi_transducer_profile_disable": [],
+    "mi_transducer_describe_plan": [_c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, ctypes.c_char_p,
+                                    _c_size_t],
     "mi_transducer_copy_probe": [_vp, _vp, _c_size_t, _vp],
 }  # fmt: skip
 
@@ -124,13 +126,27 @@ def workspace_bytes(B, T, U, D=0):
     return int(out.value)
 
 
+# pipeline stages that can be timed; which kernel runs a stage depends on the shape (describe_plan)
 PROFILE_KERNELS = {
-    "denom_gather_kernel": 0,
-    "lattice_kernel": 1,
-    "cell_kernel": 2,
-    "grad_stream_kernel": 3,
-    "zero_padding_kernel": 4,
+    "denominator_pass": 0,
+    "lattice": 1,
+    "cells": 2,
+    "gradient_pass": 3,
+    "zero_padding": 4,
 }
+
+
+def describe_plan(dtype_code, B, T, U, V, D=0, max_duration=0, use_plain_rnnt=False):
+    """{'denominators': kernel, 'lattice': kernel, 'cells': kernel or '-', 'gradient': kernel} for a shape."""
+    buf = ctypes.create_string_buffer(512)
+    check_status(
+        lib().mi_transducer_describe_plan(
+            int(dtype_code), int(B), int(T), int(U), int(V), int(D), int(max_duration), int(bool(use_plain_rnnt)),
+            buf, ctypes.c_size_t(len(buf)),
+        ),
+        "describe_plan",
+    )
+    return dict(item.split("=", 1) for item in buf.value.decode().split("; "))
 
 
 def profile_enable(max_launches, kernels=None):

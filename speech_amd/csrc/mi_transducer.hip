@@ -26,7 +26,7 @@
 
 #include <hip/hip_runtime.h>
 #include <math.h>
-#include <string.h>
+#include <stdio.h>
 #include <stdint.h>
 
 #include <vector>
@@ -2389,7 +2389,7 @@ int run_tdt_cells(const Common& c, const ScaleArg& sc, float lambda, float clamp
 // ----------------------------------------------------------------------------------------
 extern "C" {
 
-int mi_transducer_abi_version(void) { return 5; }
+int mi_transducer_abi_version(void) { return 6; }
 
 int mi_transducer_workspace_bytes(int B, int T, int U, int D, size_t* out_bytes) {
   Layout L;
@@ -2611,6 +2611,39 @@ int mi_transducer_profile_read(int kernel_id, float* total_ms, int* launches) {
 int mi_transducer_profile_disable(void) {
   g_prof.on = false;
   return MI_TRANSDUCER_SUCCESS;
+}
+
+int mi_transducer_describe_plan(int act_dtype, int B, int T, int U, int V, int D, int max_duration,
+                                int use_plain_rnnt, char* out, size_t out_bytes) {
+  Common c;
+  if (!out || out_bytes == 0 || V <= 0 || !make_layout(B, T, U, D, &c.L)) return MI_TRANSDUCER_INVALID_VALUE;
+  if (act_dtype != MI_DTYPE_F32 && act_dtype != MI_DTYPE_BF16 && act_dtype != MI_DTYPE_F16)
+    return MI_TRANSDUCER_INVALID_VALUE;
+  c.acts = nullptr; c.dt = act_dtype; c.B = B; c.T = T; c.U = U; c.V = V; c.D = D;
+  const char* dt = act_dtype == MI_DTYPE_F32 ? "f32" : (act_dtype == MI_DTYPE_BF16 ? "bf16" : "f16");
+  char denom[96], lattice[96], cells[48], grad[112];
+  const BlockPlan dp = denom_block_plan(c);
+  if (dp.RT) snprintf(denom, sizeof denom, "denom_block_kernel<%s, RT=%d, NVT=%d>", dt, dp.RT, dp.NVT);
+  else if (rows_R(c)) snprintf(denom, sizeof denom, "denom_rows_kernel<%s, R=%d>", dt, rows_R(c));
+  else snprintf(denom, sizeof denom, "denom_gather_kernel<%s>", dt);
+  const bool tdt = D > 0 && !use_plain_rnnt;
+  if (D == 0 || use_plain_rnnt) {
+    snprintf(lattice, sizeof lattice, "rnnt_lattice_kernel<K=%d>", c.L.K);
+  } else {
+    const int R = max_duration + 2;
+    const size_t lds_block = (size_t)R * 2 * D * c.L.Us * sizeof(double);
+    if (D <= 8 && c.L.Us <= 256 && lds_block <= 160 * 1024) snprintf(lattice, sizeof lattice, "tdt_lattice_block_kernel<D=%d>", D);
+    else snprintf(lattice, sizeof lattice, "tdt_lattice_kernel<K=%d>", c.L.K);
+  }
+  // a gradient buffer at the 16-byte phase of the logits is assumed (what every allocator returns)
+  const BlockPlan gp = grad_block_plan(c, nullptr);
+  const bool fused = !tdt && (gp.RT != 0 || rows_R(c) != 0);
+  snprintf(cells, sizeof cells, "%s", fused ? "-" : (tdt ? "tdt_cell_kernel" : "rnnt_cell_kernel"));
+  if (gp.RT) snprintf(grad, sizeof grad, "grad_block_kernel<%s, RT=%d, NVT=%d, %s>", dt, gp.RT, gp.NVT, fused ? "fused" : "coef");
+  else if (rows_R(c)) snprintf(grad, sizeof grad, "grad_rows_kernel<%s, R=%d, %s>", dt, rows_R(c), fused ? "fused" : "coef");
+  else snprintf(grad, sizeof grad, "grad_stream_kernel<%s>", dt);
+  const int n = snprintf(out, out_bytes, "denominators=%s; lattice=%s; cells=%s; gradient=%s", denom, lattice, cells, grad);
+  return (n < 0 || (size_t)n >= out_bytes) ? MI_TRANSDUCER_INVALID_VALUE : MI_TRANSDUCER_SUCCESS;
 }
 
 int mi_transducer_copy_probe(const void* src, void* dst, size_t bytes, void* stream) {

@@ -48,6 +48,37 @@ def test_null_and_bad_arguments_return_invalid_value_without_touching_the_gpu(bu
     assert built_lib.mi_transducer_length_maxima(None, None, 1, None, None) == 1
 
 
+def test_kernel_plan_of_the_documented_shapes(built_lib):
+    """Which kernel family a shape maps to (host logic only: nothing is launched)."""
+    F32, BF16 = 0, 1
+    plan = _native.describe_plan
+    p = plan(F32, 16, 375, 121, 1025)  # the benchmark shape: 256 whole vectors per row
+    assert p == {
+        "denominators": "denom_rows_kernel<f32, R=4>",
+        "lattice": "rnnt_lattice_kernel<K=2>",
+        "cells": "-",
+        "gradient": "grad_block_kernel<f32, RT=128, NVT=2, fused>",
+    }
+    p = plan(BF16, 32, 750, 201, 1025)  # 128 whole vectors of 8 bf16
+    assert p["denominators"] == "denom_rows_kernel<bf16, R=2>" and p["lattice"] == "rnnt_lattice_kernel<K=4>"
+    assert p["gradient"] == "grad_block_kernel<bf16, RT=64, NVT=2, fused>"
+    p = plan(F32, 8, 250, 101, 16385)  # 4096 vectors: a workgroup per row
+    assert p["denominators"] == "denom_block_kernel<f32, RT=1024, NVT=4>"
+    assert p["gradient"] == "grad_block_kernel<f32, RT=1024, NVT=4, fused>"
+    p = plan(F32, 4, 50, 21, 29)  # character vocabulary: a wave per row does everything
+    assert p["denominators"] == "denom_rows_kernel<f32, R=1>" and p["gradient"] == "grad_rows_kernel<f32, R=1, fused>"
+    p = plan(F32, 2, 10, 5, 40001)  # beyond 8 vectors per thread: the streaming kernels with a running max
+    assert p["denominators"] == "denom_gather_kernel<f32>" and p["gradient"] == "grad_stream_kernel<f32>"
+    assert p["cells"] == "rnnt_cell_kernel"
+    p = plan(F32, 16, 375, 121, 1025, D=5, max_duration=4)  # TDT: coefficients come from the cell kernel
+    assert p["lattice"] == "tdt_lattice_block_kernel<D=5>" and p["cells"] == "tdt_cell_kernel"
+    assert p["gradient"] == "grad_block_kernel<f32, RT=128, NVT=2, coef>"
+    p = plan(F32, 16, 375, 121, 1025, D=5, max_duration=4, use_plain_rnnt=True)
+    assert p["lattice"] == "rnnt_lattice_kernel<K=2>" and p["cells"] == "-"
+    with pytest.raises(RuntimeError):
+        plan(7, 1, 1, 1, 5)
+
+
 def test_constructor_attributes_match_the_reference_conventions():
     loss = RNNTLossNumba()
     assert (loss.blank, loss.reduction, loss.fastemit_lambda, loss.clamp) == (0, 'mean', 0.0, 0.0)
