@@ -879,19 +879,31 @@ __global__ __launch_bounds__(256) void tdt_lattice_block_kernel(
     for (int i = u; i < R * 2 * D * Us; i += Us) ring[i] = NEG;
     __syncthreads();
     double* out = alphas + (size_t)b * ND * Us + u;
-    double ll_acc = NEG;
-    int cur = 0;  // n % R, kept incrementally (R is a run-time value: no divisions in the loop)
+    // Ring offsets (in doubles) of the diagonals n - d_i, kept incrementally: R is a run-time value
+    // and the loop should hold no division.  The diagonal n-1-d_i of this step is the diagonal
+    // n-d_i of the previous step.
+    const int slot_stride = 2 * D * Us, ring_len = R * slot_stride;
+    int off_b[D], off_l[D];
+#pragma unroll
+    for (int i = 0; i < D; ++i) {
+      off_b[i] = ((R - dur[i]) % R) * slot_stride;
+      off_l[i] = (R - 1 - dur[i]) * slot_stride;
+    }
+    int cur_off = 0;  // offset of diagonal n's own slot
+    const int um1 = u > 0 ? u - 1 : 0;
+    // the arcs that end the utterance (t + d_i == Tb at column Ub-1, :1040-1071) are kept as they
+    // pass and summed after the loop, in the order of their steps
+    double final_arc[D];
+#pragma unroll
+    for (int i = 0; i < D; ++i) final_arc[i] = -INFINITY;
     auto step_fn = [&](int n, const float* w) {
       const int t = n - u;
       double x[2 * D];
 #pragma unroll
       for (int i = 0; i < D; ++i) {
         const int d = dur[i];
-        int sb = cur - d, sl = cur - 1 - d;  // slots of diagonals n-d and n-1-d
-        sb += sb < 0 ? R : 0;
-        sl += sl < 0 ? R : 0;
-        const double vb = ring[((sb * 2 * D) + i) * Us + u];
-        const double vl = ring[((sl * 2 * D) + D + i) * Us + (u > 0 ? u - 1 : 0)];
+        const double vb = ring[off_b[i] + i * Us + u];
+        const double vl = ring[off_l[i] + (D + i) * Us + um1];
         x[i] = (d > 0 && t >= d) ? vb : -INFINITY;
         x[D + i] = (u > 0 && t >= d) ? vl : -INFINITY;
       }
@@ -901,16 +913,21 @@ __global__ __launch_bounds__(256) void tdt_lattice_block_kernel(
       else a = lse_all(x, u == 0 ? 1 : 2);              // the emit and the no-emit accumulator are both seeded
       out[(size_t)n * Us] = a;
       const double wb = a + (double)w[0], wl = a + (double)w[1];
-      double* slot = ring + (size_t)(cur * 2 * D) * Us + u;
+      double* slot = ring + cur_off + u;
 #pragma unroll
       for (int i = 0; i < D; ++i) {
         const double dl = (double)w[2 + i];
         const double ob = (wb - sigma) + dl;
-        slot[(size_t)i * Us] = ob;
-        slot[(size_t)(D + i) * Us] = (wl - sigma) + dl;
-        if (dur[i] > 0 && u == Ub - 1 && t >= 0 && t + dur[i] == Tb) ll_acc = lse_h(ll_acc, ob);  // :1040-1071
+        slot[i * Us] = ob;
+        slot[(D + i) * Us] = (wl - sigma) + dl;
+        final_arc[i] = (dur[i] > 0 && u == Ub - 1 && t >= 0 && t + dur[i] == Tb) ? ob : final_arc[i];
       }
-      cur = cur + 1 == R ? 0 : cur + 1;
+#pragma unroll
+      for (int i = 0; i < D; ++i) {
+        off_l[i] = off_b[i];
+        off_b[i] = off_b[i] + slot_stride == ring_len ? 0 : off_b[i] + slot_stride;
+      }
+      cur_off = cur_off + slot_stride == ring_len ? 0 : cur_off + slot_stride;
       __syncthreads();
     };
     float wa[P][A], wb[P][A];
@@ -931,6 +948,11 @@ __global__ __launch_bounds__(256) void tdt_lattice_block_kernel(
       step_fn(n0, w);
     }
     if (u == Ub - 1) {
+      // a longer duration ends the utterance from an earlier diagonal: that order, as in the loop
+      double ll_acc = NEG;
+#pragma unroll
+      for (int i = D - 1; i >= 0; --i)
+        if (final_arc[i] != -INFINITY) ll_acc = lse_h(ll_acc, final_arc[i]);
       ll[2 * b] = ll_acc;
       costs[b] = -(float)ll_acc * cost_scale;
     }
@@ -939,7 +961,17 @@ __global__ __launch_bounds__(256) void tdt_lattice_block_kernel(
     __syncthreads();
     double* out = betas + (size_t)b * ND * Us + u;
     double last = NEG;
-    int cur = (nd - 1) % R;  // n % R, kept incrementally
+    // ring offsets of the diagonals n + d_i; the diagonal n+d_i+1 of this step is the diagonal
+    // n+d_i of the previous step (n runs downwards)
+    const int ring_len = R * Us;
+    int off_b[D], off_l[D];
+#pragma unroll
+    for (int i = 0; i < D; ++i) {
+      off_b[i] = (((nd - 1) % R + dur[i]) % R) * Us;
+      off_l[i] = (((nd - 1) % R + dur[i] + 1) % R) * Us;
+    }
+    int cur_off = ((nd - 1) % R) * Us;
+    const int up1 = u + 1 < Us ? u + 1 : u;
     auto step_fn = [&](int n, const float* w) {
       const int t = n - u;
       const double lpb = (double)w[0], lpl = (double)w[1];
@@ -949,11 +981,8 @@ __global__ __launch_bounds__(256) void tdt_lattice_block_kernel(
         const int d = dur[i];
         const double dl = (double)w[2 + i];
         const double bw = (lpb + dl) - sigma, lw = (lpl + dl) - sigma;
-        int sb = cur + d, sl = cur + d + 1;  // slots of diagonals n+d and n+d+1
-        sb -= sb >= R ? R : 0;
-        sl -= sl >= R ? R : 0;
-        const double vb = ring[sb * Us + u];
-        const double vl = ring[sl * Us + (u + 1 < Us ? u + 1 : u)];
+        const double vb = ring[off_b[i] + u];
+        const double vl = ring[off_l[i] + up1];
         double xb = -INFINITY;
         if (d > 0) {
           if (t + d < Tb) xb = vb + bw;
@@ -970,9 +999,14 @@ __global__ __launch_bounds__(256) void tdt_lattice_block_kernel(
       else if (t == Tb - 1 && u < Ub - 1) v = (dur[0] == 0) ? x[D] : NEG;  // last row: duration-0 labels only
       else v = lse_all(x, u == Ub - 1 ? 1 : 2);
       out[(size_t)n * Us] = v;
-      ring[cur * Us + u] = v;
+      ring[cur_off + u] = v;
       last = v;
-      cur = cur == 0 ? R - 1 : cur - 1;
+#pragma unroll
+      for (int i = 0; i < D; ++i) {
+        off_l[i] = off_b[i];
+        off_b[i] = off_b[i] == 0 ? ring_len - Us : off_b[i] - Us;
+      }
+      cur_off = cur_off == 0 ? ring_len - Us : cur_off - Us;
       __syncthreads();
     };
     float wa[P][A], wb[P][A];
