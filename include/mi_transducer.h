@@ -186,7 +186,7 @@ int mi_transducer_describe_plan(int act_dtype, int B, int T, int U, int V, int D
                                 int use_plain_rnnt, char* out, size_t out_bytes);
 
 /* Plain device-to-device copy of `bytes` (multiple of 16, 16-byte aligned pointers) with a
- * grid-stride 16-byte-per-lane kernel: the known-size yardstick for hardware traffic
+ * one-vector-per-thread kernel (the fastest streaming pattern measured): the known-size yardstick for hardware traffic
  * counters and for the copy bandwidth the GPU reaches in practice. */
 int mi_transducer_copy_probe(const void* src, void* dst, size_t bytes, void* stream);
 

@@ -2037,10 +2037,13 @@ struct ProfScope {
 
 // Plain 16-byte copy, grid-stride: the yardstick for the HBM counters and for the copy
 // bandwidth this GPU actually reaches.
+// One 16-byte vector per thread, 4 KB per workgroup, workgroups dealt to the XCDs in spans of
+// consecutive pieces: of the streaming patterns measured on this GPU (grid-stride loops, 2 to 8
+// vectors per thread, runs of pieces per workgroup) the one that copies fastest.
 __global__ __launch_bounds__(256) void copy_probe_kernel(const uint4* __restrict__ src, uint4* __restrict__ dst,
                                                          size_t nvec) {
-  const size_t stride = (size_t)gridDim.x * blockDim.x;
-  for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < nvec; i += stride) dst[i] = src[i];
+  const size_t i = (size_t)logical_block() * 256 + threadIdx.x;
+  if (i < nvec) dst[i] = src[i];
 }
 
 struct Common {
@@ -2684,8 +2687,9 @@ int mi_transducer_copy_probe(const void* src, void* dst, size_t bytes, void* str
   if (!src || !dst || bytes == 0 || (bytes & 15) || ((uintptr_t)src & 15) || ((uintptr_t)dst & 15))
     return MI_TRANSDUCER_INVALID_VALUE;
   const size_t nvec = bytes / 16;
-  size_t blocks = (nvec + 255) / 256;
-  if (blocks > 256 * 32) blocks = 256 * 32;
+  const size_t turn = 8u * MI_XCD_SPAN;
+  const size_t blocks = ((nvec + 255) / 256 + turn - 1) / turn * turn;
+  if (blocks > 0x7fffffffu) return MI_TRANSDUCER_INVALID_VALUE;
   hipLaunchKernelGGL(copy_probe_kernel, dim3((unsigned)blocks), dim3(256), 0, (hipStream_t)stream, (const uint4*)src,
                      (uint4*)dst, nvec);
   return launch_status();
