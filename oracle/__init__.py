@@ -145,3 +145,34 @@ def tdt_loss(
         denom=denom, dlp=dlp, alphas=alphas, betas=betas, ll_forward=llf, ll_backward=llb, duration_grads=dgrads_lp
     )
     return costs, grads, extras
+
+
+def multiblank_loss(
+    acts, labels, act_lens, label_lens, blank, big_blank_durations, sigma=0.0, fastemit_lambda=0.0, clamp=0.0,
+    dtype=np.float64, want_grads=True, num_threads=1,
+):  # fmt: skip
+    """Multi-blank transducer, GPU-path semantics.  Returns (costs, grads or None, extras)."""
+    suf, creal = _real(dtype)
+    acts, labels, act_lens, label_lens = _prep(acts, labels, act_lens, label_lens, dtype)
+    durations = np.ascontiguousarray(big_blank_durations, dtype=np.int32)
+    NB = int(durations.shape[0])
+    B, T, U, V = acts.shape
+    costs = np.zeros(B, dtype=dtype)
+    grads = np.zeros_like(acts) if want_grads else None
+    denom = np.zeros((B, T, U), dtype=dtype)
+    alphas = np.full((B, T, U), -np.inf, dtype=dtype)
+    betas = np.full((B, T, U), -np.inf, dtype=dtype)
+    llf = np.zeros(B, dtype=dtype)
+    llb = np.zeros(B, dtype=dtype)
+    fn = getattr(lib(), "oracle_multiblank_loss_" + suf)
+    fn.restype = ctypes.c_int
+    status = fn(
+        _ptr(acts), _ptr(labels), _ptr(act_lens), _ptr(label_lens),
+        ctypes.c_int(B), ctypes.c_int(T), ctypes.c_int(U), ctypes.c_int(V), ctypes.c_int(NB),
+        _ptr(durations) if NB else None, ctypes.c_int(blank), creal(sigma), creal(fastemit_lambda), creal(clamp),
+        _ptr(costs), _ptr(grads), _ptr(denom), _ptr(alphas), _ptr(betas), _ptr(llf), _ptr(llb),
+        ctypes.c_int(num_threads),
+    )  # fmt: skip
+    if status != 0:
+        raise RuntimeError("oracle_multiblank_loss: invalid value")
+    return costs, grads, dict(denom=denom, alphas=alphas, betas=betas, ll_forward=llf, ll_backward=llb)

@@ -12,11 +12,15 @@
  *                                   sparse log-prob gradient, softmax Jacobian, clamp hook);
  *                                   this is the timed CPU baseline
  *   oracle_tdt_loss_{f32,f64}       TDT, GPU-path semantics (the reference has no CPU TDT)
+ *   oracle_multiblank_loss_{f32,f64}  multi-blank transducer, GPU-path semantics (no CPU path
+ *                                   in the reference either)
  *
  * Pinning: every entry point is checked against the reference's golden vectors
  * and against oracle/transducer_numpy.py, brute-force path enumeration and torch
  * autograd in tests/test_oracle_*.py.  TDT with FastEmit has no reference vector:
- * it is checked only against the sparse-posterior identity ("derived").
+ * it is checked only against the sparse-posterior identity ("derived").  The reference holds no
+ * vector for the multi-blank loss: it is pinned by the RNNT vectors (no big blank, sigma 0),
+ * path enumeration and autograd; its FastEmit terms are "derived" too.
  *
  * Build: make -C oracle   (gcc -O2 -fopenmp, no fast-math so the operation order stands)
  */

@@ -18,6 +18,13 @@ How each function is pinned (tests/test_oracle_*.py):
                     torch autograd, T=1 and U=1 closed forms ......... pinned
   tdt_* FastEmit    no reference vector exists; checked only against the
                     sparse-posterior + softmax-Jacobian identity ..... derived
+  multiblank_*      the reference holds no vector (its test compares two of
+                    its own implementations on random input); with no big
+                    blank and sigma = 0 it must give the RNNT golden vectors,
+                    brute-force enumeration of every (token, blank-duration)
+                    path, torch autograd of an alpha-only recursion,
+                    llForward == beta(0,0) ........................... pinned
+  multiblank_* FastEmit  derived only, as for TDT
 
 The loops are slow on purpose (clarity first): use them at lattice sizes up to
 a few thousand cells; oracle/transducer_cpu.c is the fast restatement.
@@ -418,3 +425,141 @@ def tdt_loss(
         duration_grads=duration_grads,
     )
     return costs, grads, extras
+
+
+# ----------------------------------------------------------------------------
+# Multi-blank transducer (utils/cuda_utils/gpu_rnnt_kernel.py:410-885)
+# ----------------------------------------------------------------------------
+# The softmax runs over V token logits, then the big blanks, then the standard blank: big blank i
+# (duration big_blank_durations[i]) sits at index blank-1-i.  Every arc score is lp - sigma.
+
+
+def multiblank_alphas(lp, labels, T, U, blank, big_blank_durations, sigma):
+    """Forward variables; gpu_rnnt_kernel.py:410-568.  Returns (alphas[T,U], llForward)."""
+    dt = lp.dtype.type
+    sig = dt(sigma)
+    a = np.full((T, U), NEG_INF, dtype=lp.dtype)
+    a[0, 0] = dt(0)
+    for t in range(T):
+        for u in range(U):
+            if t == 0 and u == 0:
+                continue
+            if u == 0:
+                acc = a[t - 1, 0] + lp[t - 1, 0, blank] - sig
+                for i, d in enumerate(big_blank_durations):
+                    if t >= d:
+                        acc = lse2(acc, a[t - d, 0] + lp[t - d, 0, blank - 1 - i] - sig)
+                a[t, 0] = acc
+            elif t == 0:
+                a[0, u] = a[0, u - 1] + lp[0, u - 1, labels[u - 1]] - sig
+            else:
+                no_emit = a[t - 1, u] + lp[t - 1, u, blank] - sig
+                emit = a[t, u - 1] + lp[t, u - 1, labels[u - 1]] - sig
+                acc = lse2(emit, no_emit)
+                for i, d in enumerate(big_blank_durations):
+                    if t >= d:
+                        acc = lse2(acc, a[t - d, u] + lp[t - d, u, blank - 1 - i] - sig)
+                a[t, u] = acc
+    ll = a[T - 1, U - 1] + lp[T - 1, U - 1, blank] - sig
+    for i, d in enumerate(big_blank_durations):
+        if T >= d:
+            ll = lse2(ll, a[T - d, U - 1] + lp[T - d, U - 1, blank - 1 - i] - sig)
+    return a, ll
+
+
+def multiblank_betas(lp, labels, T, U, blank, big_blank_durations, sigma):
+    """Backward variables; gpu_rnnt_kernel.py:571-724.  Returns (betas[T,U], llBackward)."""
+    dt = lp.dtype.type
+    sig = dt(sigma)
+    bt = np.full((T, U), NEG_INF, dtype=lp.dtype)
+    bt[T - 1, U - 1] = lp[T - 1, U - 1, blank] - sig
+    for t in range(T - 1, -1, -1):
+        for u in range(U - 1, -1, -1):
+            if t == T - 1 and u == U - 1:
+                continue
+            if u == U - 1:
+                acc = bt[t + 1, U - 1] + lp[t, U - 1, blank] - sig
+                for i, d in enumerate(big_blank_durations):
+                    if t + d < T:
+                        acc = lse2(acc, bt[t + d, U - 1] + lp[t, U - 1, blank - 1 - i] - sig)
+                    elif t + d == T and d != 1:
+                        acc = lse2(acc, lp[t, U - 1, blank - 1 - i] - sig)
+                bt[t, U - 1] = acc
+            elif t == T - 1:
+                bt[T - 1, u] = bt[T - 1, u + 1] + lp[T - 1, u, labels[u]] - sig
+            else:
+                no_emit = bt[t + 1, u] + lp[t, u, blank] - sig
+                emit = bt[t, u + 1] + lp[t, u, labels[u]] - sig
+                acc = lse2(emit, no_emit)
+                for i, d in enumerate(big_blank_durations):
+                    if t < T - d:
+                        acc = lse2(acc, bt[t + d, u] + lp[t, u, blank - 1 - i] - sig)
+                bt[t, u] = acc
+    return bt, bt[0, 0]
+
+
+def multiblank_grads(lp, alphas, betas, ll, labels, T, U, blank, big_blank_durations, sigma, fastemit_lambda, clamp):
+    """Gradient w.r.t. the logits for the valid cells; gpu_rnnt_kernel.py:727-885."""
+    dt = lp.dtype.type
+    sig = dt(sigma)
+    lam = dt(fastemit_lambda)
+    V = lp.shape[-1]
+    g = np.zeros((T, U, V), dtype=lp.dtype)
+    for t in range(T):
+        for u in range(U):
+            row = np.exp(alphas[t, u] + betas[t, u] + lp[t, u, :] - ll)
+            if fastemit_lambda > 0.0 and u < U - 1:
+                row = row + lam * np.exp(
+                    alphas[t, u] + lp[t, u, labels[u]] + betas[t, u + 1] + lp[t, u, :] - sig - ll
+                )
+            if t == T - 1 and u == U - 1:
+                row[blank] -= np.exp(alphas[t, u] + lp[t, u, blank] - sig - ll)
+            for i, d in enumerate(big_blank_durations):
+                k = blank - 1 - i
+                if t == T - d and u == U - 1:
+                    row[k] -= np.exp(alphas[t, u] + lp[t, u, k] - sig - ll)
+            if t < T - 1:
+                row[blank] -= np.exp(alphas[t, u] + lp[t, u, blank] - sig - ll + betas[t + 1, u])
+            for i, d in enumerate(big_blank_durations):
+                k = blank - 1 - i
+                if t < T - d:
+                    row[k] -= np.exp(alphas[t, u] + lp[t, u, k] - sig - ll + betas[t + d, u])
+            if u < U - 1:
+                v = labels[u]
+                row[v] -= np.exp(np.log1p(lam) + alphas[t, u] + lp[t, u, v] - sig - ll + betas[t, u + 1])
+            if clamp > 0.0:
+                row = np.minimum(np.maximum(row, dt(-clamp)), dt(clamp))
+            g[t, u, :] = row
+    return g
+
+
+def multiblank_loss(
+    acts, labels, act_lens, label_lens, blank, big_blank_durations, sigma=0.0, fastemit_lambda=0.0, clamp=0.0,
+    dtype=np.float64,
+):  # fmt: skip
+    """Per-utterance costs and logits-gradient; MultiblankGPURNNT.compute_cost_and_score
+    (utils/cuda_utils/gpu_rnnt.py:343-440) + compute_costs_data (utils/rnnt_helper.py:106-116).
+    `acts` are raw logits [B,T,U,V_tokens + num_big_blanks + 1]."""
+    acts = np.asarray(acts, dtype=dtype)
+    B, Tm, Um, V = acts.shape
+    denom = denominator(acts)
+    costs = np.zeros(B, dtype=dtype)
+    grads = np.zeros_like(acts)
+    alphas = np.full((B, Tm, Um), NEG_INF, dtype=dtype)
+    betas = np.full((B, Tm, Um), NEG_INF, dtype=dtype)
+    llf = np.zeros(B, dtype=dtype)
+    llb = np.zeros(B, dtype=dtype)
+    durs = [int(d) for d in big_blank_durations]
+    for b in range(B):
+        T = int(act_lens[b])
+        U = int(label_lens[b]) + 1
+        lp = acts[b] + denom[b][..., None]
+        lab = [int(x) for x in labels[b][: U - 1]]
+        a, ll = multiblank_alphas(lp, lab, T, U, blank, durs, sigma)
+        bt, ll_b = multiblank_betas(lp, lab, T, U, blank, durs, sigma)
+        grads[b, :T, :U, :] = multiblank_grads(lp, a, bt, ll, lab, T, U, blank, durs, sigma, fastemit_lambda, clamp)
+        alphas[b, :T, :U] = a
+        betas[b, :T, :U] = bt
+        llf[b], llb[b] = ll, ll_b
+        costs[b] = -ll * dtype(1.0 + fastemit_lambda)
+    return costs, grads, dict(denom=denom, alphas=alphas, betas=betas, ll_forward=llf, ll_backward=llb)

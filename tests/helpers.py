@@ -166,3 +166,62 @@ def tdt_autograd(logits, labels, blank, durations, sigma, lam=0.0):
     g_tok = g_blank + (1.0 + lam) * g_lab
     torch.autograd.backward([lp, dlp], [g_tok, g_dur])
     return float(nll.detach()) * (1.0 + lam), x.grad.numpy()
+
+
+def multiblank_bruteforce_ll(logits, labels, blank, big_blank_durations, sigma):
+    """Multi-blank log-likelihood (arXiv:2211.03541) by enumerating every path.  logits: [T,U,V]
+    float64 with one softmax over tokens, big blanks (index blank-1-i, duration d_i) and the standard
+    blank (duration 1); every arc pays -sigma.  A label stays on the frame; a blank of duration d
+    moves to frame t+d, which must exist unless the path ends there (t+d == T at u == U-1)."""
+    T, U, _ = logits.shape
+    lp = logits - np.log(np.exp(logits).sum(-1, keepdims=True))
+    blanks = [(blank, 1)] + [(blank - 1 - i, d) for i, d in enumerate(big_blank_durations)]
+    totals = []
+
+    def walk(t, u, acc):
+        for k, d in blanks:
+            w = acc + lp[t, u, k] - sigma
+            if t + d < T:
+                walk(t + d, u, w)
+            elif t + d == T and u == U - 1:
+                totals.append(w)
+        if u < U - 1:
+            walk(t, u + 1, acc + lp[t, u, labels[u]] - sigma)
+
+    walk(0, 0, 0.0)
+    return logsumexp_list(totals)
+
+
+def multiblank_autograd(logits, labels, blank, big_blank_durations, sigma, lam=0.0):
+    """(-ll, d(-ll)/dlogits) for the multi-blank transducer from an alpha-only recursion in torch
+    float64.  With lam > 0 the log-prob gradient entries of label arcs are scaled by (1+lam) before
+    the log-softmax Jacobian and the cost by (1+lam): what the kernel's FastEmit terms amount to."""
+    x = torch.tensor(np.asarray(logits, dtype=np.float64), requires_grad=True)
+    T, U, _ = x.shape
+    lp = torch.log_softmax(x, dim=-1)
+    lp_blank = lp.detach().clone().requires_grad_(True)
+    lp_lab = lp.detach().clone().requires_grad_(True)
+    blanks = [(blank, 1)] + [(blank - 1 - i, d) for i, d in enumerate(big_blank_durations)]
+    alpha = [[None] * U for _ in range(T)]
+    alpha[0][0] = torch.zeros((), dtype=torch.float64)
+    for t in range(T):
+        for u in range(U):
+            if t == 0 and u == 0:
+                continue
+            terms = []
+            for k, d in blanks:
+                if t - d >= 0 and alpha[t - d][u] is not None:
+                    terms.append(alpha[t - d][u] + lp_blank[t - d, u, k] - sigma)
+            if u > 0 and alpha[t][u - 1] is not None:
+                terms.append(alpha[t][u - 1] + lp_lab[t, u - 1, labels[u - 1]] - sigma)
+            alpha[t][u] = torch.logsumexp(torch.stack(terms), dim=0) if terms else None
+    finals = [
+        alpha[T - d][U - 1] + lp_blank[T - d, U - 1, k] - sigma
+        for k, d in blanks
+        if T - d >= 0 and alpha[T - d][U - 1] is not None
+    ]
+    nll = -torch.logsumexp(torch.stack(finals), dim=0)
+    g_blank, g_lab = torch.autograd.grad(nll, [lp_blank, lp_lab], allow_unused=True)
+    g_lab = torch.zeros_like(lp) if g_lab is None else g_lab
+    lp.backward(g_blank + (1.0 + lam) * g_lab)
+    return float(nll.detach()) * (1.0 + lam), x.grad.numpy()
