@@ -4,6 +4,7 @@
  * runs below its function-level seam (nemo/collections/asr/parts/numba/rnnt_loss/):
  *   rnnt.py:138-236  rnnt_loss_gpu      -> mi_rnnt_loss  (or mi_rnnt_forward + mi_rnnt_backward)
  *   rnnt.py:239-363  tdt_loss_gpu       -> mi_tdt_loss   (or mi_tdt_forward  + mi_tdt_backward)
+ *   rnnt.py:366-483  multiblank_rnnt_loss_gpu -> mi_multiblank_loss (or _forward + _backward)
  *   utils/rnnt_helper.py:119-142 get_workspace_size -> mi_transducer_workspace_bytes
  *
  * Conventions
@@ -45,6 +46,8 @@ extern "C" {
 
 #define MI_TRANSDUCER_MAX_U 1024
 #define MI_TRANSDUCER_MAX_DURATIONS 16
+#define MI_TRANSDUCER_MAX_BIG_BLANKS 8      /* multi-blank: big blanks beside the standard blank */
+#define MI_TRANSDUCER_MAX_BLANK_DURATION 64 /* multi-blank: longest big-blank duration */
 
 /* Library/ABI version; bumped whenever a signature below changes. */
 int mi_transducer_abi_version(void);
@@ -116,6 +119,33 @@ int mi_tdt_loss(const void* acts, int act_dtype, const int64_t* labels, const in
                 float grad_mul, int B, int T, int U, int V, int D, const int32_t* durations_host, int blank,
                 float fastemit_lambda, float clamp, float sigma, int use_plain_rnnt, void* workspace,
                 size_t workspace_bytes, void* stream);
+
+/* ---- multi-blank transducer ---------------------------------------------------------
+ * Replaces rnnt.py:366-483 (multiblank_rnnt_loss_gpu) and what it drives:
+ * gpu_rnnt.py:296-509 (MultiblankGPURNNT), gpu_rnnt_kernel.py:410-885 (alphas, betas, gradient).
+ * acts: [B,T,U,V] raw logits where V counts the tokens, the num_big_blanks big blanks and the
+ * standard blank; big blank i (duration big_blank_durations_host[i] >= 1 frames, host int32
+ * array) sits at index blank-1-i; one softmax covers all V entries and every arc pays -sigma.
+ * workspace: mi_transducer_workspace_bytes(B, T, U, num_big_blanks).  num_big_blanks <=
+ * MI_TRANSDUCER_MAX_BIG_BLANKS, durations <= MI_TRANSDUCER_MAX_BLANK_DURATION, and the LDS ring
+ * (longest duration + 1) * (2 + capacity) * 64*ceil(U/64) * 8 bytes must fit 160 KB (capacity =
+ * num_big_blanks rounded up to 1, 2, 4 or 8), else invalid value.  Other arguments as for RNNT. */
+int mi_multiblank_forward(const void* acts, int act_dtype, const int64_t* labels, const int64_t* act_lens,
+                          const int64_t* label_lens, float* costs, int B, int T, int U, int V, int num_big_blanks,
+                          const int32_t* big_blank_durations_host, int blank, float fastemit_lambda, float sigma,
+                          int with_betas, void* workspace, size_t workspace_bytes, void* stream);
+
+int mi_multiblank_backward(const void* acts, int act_dtype, const int64_t* labels, const int64_t* act_lens,
+                           const int64_t* label_lens, void* grads, const float* grad_scale, int grad_scale_stride,
+                           float grad_mul, int B, int T, int U, int V, int num_big_blanks,
+                           const int32_t* big_blank_durations_host, int blank, float fastemit_lambda, float clamp,
+                           float sigma, void* workspace, size_t workspace_bytes, void* stream);
+
+int mi_multiblank_loss(const void* acts, int act_dtype, const int64_t* labels, const int64_t* act_lens,
+                       const int64_t* label_lens, float* costs, void* grads, const float* grad_scale,
+                       int grad_scale_stride, float grad_mul, int B, int T, int U, int V, int num_big_blanks,
+                       const int32_t* big_blank_durations_host, int blank, float fastemit_lambda, float clamp,
+                       float sigma, void* workspace, size_t workspace_bytes, void* stream);
 
 /* The two stages of a forward call on their own (mi_rnnt_forward = denominators + rnnt lattice,
  * mi_tdt_forward = denominators + tdt lattice), for callers that want to order other work between

@@ -398,7 +398,7 @@ template <int DT>
 __global__ __launch_bounds__(256) void denom_gather_kernel(
     const void* __restrict__ acts, const int64_t* __restrict__ labels, const int64_t* __restrict__ act_lens,
     const int64_t* __restrict__ label_lens, float* __restrict__ denom, float* __restrict__ arcs, int T, int U, int V,
-    int D, int blank, int ND, int Us, int A, int BT, int bt_chunk) {
+    int D, int nbig, int blank, int ND, int Us, int A, int BT, int bt_chunk) {
   constexpr int VEC = Elem<DT>::VEC;
   constexpr int R = 4;  // vectors in flight per lane
   constexpr bool NT = MI_NT_K1 != 0;
@@ -417,7 +417,8 @@ __global__ __launch_bounds__(256) void denom_gather_kernel(
   const int lab = (u < Ub - 1) ? clampi(labels[(size_t)b * (U - 1) + u], 0, V - 1) : -1;
   const float xb = Elem<DT>::load1(acts, e0 + blank);
   const float xl = Elem<DT>::load1(acts, e0 + (lab >= 0 ? lab : blank));
-  const float xd = (lane < D) ? Elem<DT>::load1(acts, e0 + V + lane) : kNegInf;
+  const float xd = (lane < D) ? Elem<DT>::load1(acts, e0 + V + lane)
+                              : (lane < nbig ? Elem<DT>::load1(acts, e0 + blank - 1 - lane) : kNegInf);
 
   const RowWindow<DT> w(acts, e0);
   const RowSplit<DT> sp(w.mis, V);
@@ -468,6 +469,7 @@ __global__ __launch_bounds__(256) void denom_gather_kernel(
     const float dden = -dm - logf(ds);
     if (lane < D) arcs[base + (size_t)(2 + lane) * Us] = xd + dden;
   }
+  if (lane < nbig) arcs[base + (size_t)(2 + lane) * Us] = xd + dn;  // big-blank log-probs (multi-blank)
 }
 
 // ----------------------------------------------------------------------------------------
@@ -1253,6 +1255,258 @@ __global__ __launch_bounds__(256) void tdt_cell_kernel(
 }
 
 // ----------------------------------------------------------------------------------------
+// Multi-blank transducer (arXiv:2211.03541; gpu_rnnt_kernel.py:410-724).  The softmax covers the
+// tokens, NB big blanks (big blank i: index blank-1-i, duration dur[i]) and the standard blank
+// (duration 1); every arc pays -sigma.  Same organisation as the TDT workgroup kernel: one
+// workgroup per (utterance, direction), one thread per column, one barrier per anti-diagonal.
+//   alpha: a finished cell leaves alpha + arc - sigma for each of its outgoing arcs in an LDS
+//          ring of max_duration + 1 diagonals (plane 0: label arc, read by column u+1 one step
+//          later; plane 1+j: blank arc j, read by the same column dur_j steps later).
+//   beta : the ring holds beta of the last max_duration + 1 diagonals.
+// Cells outside the lattice hold "log 0" or junk that no valid cell reads, as in the RNNT kernel.
+// NBC is the compiled capacity for big blanks; prm.NB <= NBC are in use.
+// ----------------------------------------------------------------------------------------
+struct MbParams {
+  int NB;
+  int dur[MI_TRANSDUCER_MAX_BIG_BLANKS];
+  int R;  // ring depth: longest blank + 1
+  float sigma;
+};
+
+template <int NBC>
+__global__ __launch_bounds__(1024) void multiblank_lattice_kernel(
+    const float* __restrict__ arcs, double* __restrict__ alphas, double* __restrict__ betas, double* __restrict__ ll,
+    float* __restrict__ costs, const int64_t* __restrict__ act_lens, const int64_t* __restrict__ label_lens, int T,
+    int U, int ND, int Us, int A, float cost_scale, int with_betas, MbParams prm) {
+  constexpr int P = 4;
+  constexpr int NJ = NBC + 1;  // blank arcs: the standard one, then the big ones
+  extern __shared__ double ring[];
+  const int b = with_betas ? (int)(blockIdx.x >> 1) : (int)blockIdx.x;
+  const int dir = with_betas ? (int)(blockIdx.x & 1) : 0;
+  const int u = threadIdx.x;  // blockDim.x == Us
+  const int Tb = clampi(act_lens[b], 1, T);
+  const int Ub = clampi(label_lens[b] + 1, 1, U);
+  const int nd = Tb + Ub - 1;
+  const int R = prm.R, NB = prm.NB;
+  const double sigma = (double)prm.sigma;
+  const double NINF = kLogZero;
+  int dur[NJ];
+  dur[0] = 1;
+#pragma unroll
+  for (int j = 1; j < NJ; ++j) dur[j] = j - 1 < NB ? prm.dur[j - 1] : (1 << 28);  // unused slots never fire
+  const size_t row_pitch = (size_t)A * Us;
+  const float* arcs_b = arcs + (size_t)b * ND * row_pitch + u;
+
+  // arc log-probs of P diagonals for this column: [0] standard blank, [1] label, [2+i] big blank i
+  auto load_rows = [&](int nfirst, int step, float(&W)[P][2 + NBC]) {
+#pragma unroll
+    for (int p = 0; p < P; ++p) {
+      int n = nfirst + step * p;
+      n = n < 0 ? 0 : (n >= nd ? nd - 1 : n);
+      const float* rp = arcs_b + (size_t)n * row_pitch;
+      W[p][0] = finite_arc(rp[0]);
+      W[p][1] = finite_arc(rp[Us]);
+#pragma unroll
+      for (int i = 0; i < NBC; ++i) W[p][2 + i] = i < NB ? finite_arc(rp[(size_t)(2 + i) * Us]) : 0.f;
+    }
+  };
+  // log-sum-exp of x[0..N); "log 0" entries vanish, all "log 0" stays "log 0"
+  auto lse_all = [&](const double* x) {
+    constexpr int N = 1 + NJ;
+    double m = x[0];
+#pragma unroll
+    for (int i = 1; i < N; ++i) m = fmax(m, x[i]);
+    float s = 0.f;
+#pragma unroll
+    for (int i = 0; i < N; ++i) s += fast_exp2((float)(x[i] - m) * kLog2e);
+    return m + (double)(__builtin_amdgcn_logf(s) * 0.6931471805599453f);
+  };
+
+  if (dir == 0) {
+    const int slot_stride = (1 + NJ) * Us, ring_len = R * slot_stride;
+    for (int i = u; i < ring_len; i += Us) ring[i] = NINF;
+    __syncthreads();
+    double* out = alphas + (size_t)b * ND * Us + u;
+    // ring offsets of the diagonals n-1 (label arc, standard blank) and n-dur_j (big blanks)
+    int off_in[NJ];
+#pragma unroll
+    for (int j = 0; j < NJ; ++j) off_in[j] = j - 1 < NB ? ((R - dur[j] % R) % R) * slot_stride : 0;
+    int cur_off = 0;
+    const int um1 = u > 0 ? u - 1 : 0;
+    // arcs that end the utterance (column Ub-1, t + dur_j == Tb), kept as they pass; gpu_rnnt_kernel.py:548-568
+    double final_arc[NJ];
+#pragma unroll
+    for (int j = 0; j < NJ; ++j) final_arc[j] = NINF;
+    auto step_fn = [&](int n, const float* w) {
+      const int t = n - u;
+      double x[1 + NJ];
+      x[0] = u > 0 ? ring[off_in[0] + um1] : NINF;  // label arc out of (t, u-1)
+#pragma unroll
+      for (int j = 0; j < NJ; ++j) x[1 + j] = ring[off_in[j] + (1 + j) * Us + u];  // blank arc j out of (t-dur_j, u)
+      double a = lse_all(x);
+      if (n == 0 && u == 0) a = 0.0;
+      out[(size_t)n * Us] = a;
+      double* slot = ring + cur_off + u;
+      slot[0] = (a + (double)w[1]) - sigma;
+#pragma unroll
+      for (int j = 0; j < NJ; ++j) {
+        const double ob = (a + (double)w[j == 0 ? 0 : 1 + j]) - sigma;
+        slot[(1 + j) * Us] = j - 1 < NB ? ob : NINF;
+        final_arc[j] = (j - 1 < NB && u == Ub - 1 && t >= 0 && t + dur[j] == Tb) ? ob : final_arc[j];
+      }
+#pragma unroll
+      for (int j = 0; j < NJ; ++j) off_in[j] = off_in[j] + slot_stride == ring_len ? 0 : off_in[j] + slot_stride;
+      cur_off = cur_off + slot_stride == ring_len ? 0 : cur_off + slot_stride;
+      __syncthreads();
+    };
+    float wa[P][2 + NBC], wb[P][2 + NBC];
+    int n0 = 0;
+    load_rows(0, 1, wa);
+    for (; n0 + 2 * P <= nd; n0 += 2 * P) {
+      load_rows(n0 + P, 1, wb);
+#pragma unroll
+      for (int p = 0; p < P; ++p) step_fn(n0 + p, wa[p]);
+      load_rows(n0 + 2 * P, 1, wa);
+#pragma unroll
+      for (int p = 0; p < P; ++p) step_fn(n0 + P + p, wb[p]);
+    }
+    for (; n0 < nd; ++n0) {
+      float w[P][2 + NBC];
+      load_rows(n0, 0, w);
+      step_fn(n0, w[0]);
+    }
+    if (u == Ub - 1) {
+      // the standard blank first, then the big blanks in their order (gpu_rnnt_kernel.py:548-568)
+      double acc = final_arc[0];
+#pragma unroll
+      for (int j = 1; j < NJ; ++j) acc = lse_h(acc, final_arc[j]);
+      ll[2 * b] = acc;
+      costs[b] = -(float)acc * cost_scale;
+    }
+  } else {
+    const int ring_len = R * Us;
+    for (int i = u; i < ring_len; i += Us) ring[i] = NINF;
+    __syncthreads();
+    double* out = betas + (size_t)b * ND * Us + u;
+    double last = NINF;
+    // ring offsets of the diagonals n+dur_j; the label arc reads diagonal n+1 like the standard blank
+    int off_in[NJ];
+#pragma unroll
+    for (int j = 0; j < NJ; ++j) off_in[j] = j - 1 < NB ? (((nd - 1) % R + dur[j] % R) % R) * Us : 0;
+    int cur_off = ((nd - 1) % R) * Us;
+    const int up1 = u + 1 < Us ? u + 1 : u;
+    auto step_fn = [&](int n, const float* w) {
+      const int t = n - u;
+      double x[1 + NJ];
+      x[0] = (t < Tb && u < Ub - 1) ? (ring[off_in[0] + up1] + (double)w[1]) - sigma : NINF;  // label arc to (t, u+1)
+#pragma unroll
+      for (int j = 0; j < NJ; ++j) {
+        const double arc = (double)w[j == 0 ? 0 : 1 + j] - sigma;
+        double xb = NINF;
+        if (j - 1 < NB) {
+          if (t + dur[j] < Tb) xb = ring[off_in[j] + u] + arc;
+          // a big blank may end the utterance from column Ub-1 (gpu_rnnt_kernel.py:660-670; the standard
+          // blank does so through the corner cell)
+          else if (j > 0 && t + dur[j] == Tb && u == Ub - 1 && dur[j] != 1) xb = arc;
+        }
+        x[1 + j] = xb;
+      }
+      double v = lse_all(x);
+      if (t == Tb - 1 && u == Ub - 1) v = (double)w[0] - sigma;  // the corner: one standard blank
+      out[(size_t)n * Us] = v;
+      ring[cur_off + u] = v;
+      last = v;
+#pragma unroll
+      for (int j = 0; j < NJ; ++j) off_in[j] = off_in[j] == 0 ? ring_len - Us : off_in[j] - Us;
+      cur_off = cur_off == 0 ? ring_len - Us : cur_off - Us;
+      __syncthreads();
+    };
+    float wa[P][2 + NBC], wb[P][2 + NBC];
+    int n0 = nd - 1;
+    load_rows(n0, -1, wa);
+    for (; n0 - 2 * P + 1 >= 0; n0 -= 2 * P) {
+      load_rows(n0 - P, -1, wb);
+#pragma unroll
+      for (int p = 0; p < P; ++p) step_fn(n0 - p, wa[p]);
+      load_rows(n0 - 2 * P, -1, wa);
+#pragma unroll
+      for (int p = 0; p < P; ++p) step_fn(n0 - P - p, wb[p]);
+    }
+    for (; n0 >= 0; --n0) {
+      float w[P][2 + NBC];
+      load_rows(n0, 0, w);
+      step_fn(n0, w[0]);
+    }
+    if (u == 0) ll[2 * b + 1] = last;  // beta(0,0)
+  }
+}
+
+// Per-cell coefficients of the multi-blank gradient (gpu_rnnt_kernel.py:727-885): the record of the
+// RNNT/TDT cell kernels, plus in out[kCoefBase + i] the FINISHED gradient entry of big blank i
+// (clamped and scaled), which multiblank_fixup_kernel stores over what the gradient pass put there.
+__global__ __launch_bounds__(256) void multiblank_cell_kernel(
+    const float* __restrict__ denom, const float* __restrict__ arcs,
+    const double* __restrict__ alphas, const double* __restrict__ betas, const double* __restrict__ ll,
+    const int64_t* __restrict__ labels, const int64_t* __restrict__ act_lens, const int64_t* __restrict__ label_lens,
+    const float* __restrict__ grad_scale, int grad_scale_stride, float grad_mul, float* __restrict__ coef, int T, int U,
+    int V, int blank, int ND, int Us, int A, int CS, float lambda, float clamp, long long cells, MbParams prm) {
+  const long long c = (long long)blockIdx.x * blockDim.x + threadIdx.x;
+  if (c >= cells) return;
+  const int u = (int)(c % U);
+  const long long bt = c / U;
+  const int t = (int)(bt % T);
+  const int b = (int)(bt / T);
+  const int Tb = clampi(act_lens[b], 1, T);
+  const int Ub = clampi(label_lens[b] + 1, 1, U);
+  float* out = coef + (size_t)c * CS;
+  if (t >= Tb || u >= Ub) {
+    out[5] = __int_as_float(-2);
+    return;
+  }
+  const double sigma = (double)prm.sigma;
+  const size_t row = (size_t)(b * ND + t + u);
+  const size_t sk = row * Us + u;
+  const double a = alphas[sk], bb = betas[sk], L = ll[2 * b];
+  const float* rp = arcs + row * A * Us + u;
+  const float lpb = rp[0], lpl = rp[Us];
+  const int lab = (u < Ub - 1) ? clampi(labels[(size_t)b * (U - 1) + u], 0, V - 1) : -1;
+  const float scale = (grad_scale ? grad_scale[(size_t)b * grad_scale_stride] : 1.f) * grad_mul;
+  const float gamma = expf((float)(a + bb - L));
+  float pb = 0.f, pl = 0.f;
+  if (t < Tb - 1) pb = expf((float)(a + betas[sk + Us] + (double)lpb - sigma - L));
+  else if (u == Ub - 1) pb = expf((float)(a + (double)lpb - sigma - L));
+  if (lab >= 0) pl = expf((float)(a + betas[sk + Us + 1] + (double)lpl - sigma - L));
+  const float W = gamma + lambda * pl, PL = (1.f + lambda) * pl;
+#pragma unroll 1
+  for (int i = 0; i < prm.NB; ++i) {
+    const int d = prm.dur[i];
+    const float lpi = rp[(size_t)(2 + i) * Us];
+    float pi = 0.f;
+    if (t + d < Tb) pi = expf((float)(a + betas[sk + (size_t)d * Us] + (double)lpi - sigma - L));
+    else if (t + d == Tb && u == Ub - 1) pi = expf((float)(a + (double)lpi - sigma - L));
+    float g = expf(lpi) * W - pi;
+    if (lab == blank - 1 - i) g -= PL;
+    if (clamp > 0.f) g = clamp_sym(g, clamp);
+    out[kCoefBase + i] = g * scale;
+  }
+  write_coef(out, make_coef(denom[c], W, pb, PL, lpb, lpl, lab, blank, clamp, scale));
+}
+
+// stores the finished big-blank entries of every valid cell (after the gradient pass)
+template <int DT>
+__global__ __launch_bounds__(256) void multiblank_fixup_kernel(void* __restrict__ grads, const float* __restrict__ coef,
+                                                               int V, int blank, int NB, int CS, long long cells) {
+  const long long i = (long long)blockIdx.x * blockDim.x + threadIdx.x;
+  const long long c = i / NB;
+  if (c >= cells) return;
+  const int k = (int)(i - c * NB);
+  const float* rec = coef + (size_t)c * CS;
+  if (__float_as_int(rec[5]) == -2) return;  // padded cell
+  Elem<DT>::store1(grads, (size_t)c * V + (blank - 1 - k), rec[kCoefBase + k]);
+}
+
+
+// ----------------------------------------------------------------------------------------
 // Pass 2: the gradient stream.  Grid (ceil(U/4), T, B), one wave per row; reads the V token
 // logits of valid rows, writes V + D gradient elements of every row.  Same kernel for RNNT
 // (D = 0) and TDT.  flags: kFlagZeroDurations, kFlagPaddingDone.
@@ -1435,12 +1689,12 @@ template <int DT, int R>
 __global__ __launch_bounds__(kRowThreads) void denom_rows_kernel(
     const void* __restrict__ acts, const int64_t* __restrict__ labels, const int64_t* __restrict__ act_lens,
     const int64_t* __restrict__ label_lens, float* __restrict__ denom, float* __restrict__ arcs, int T, int U, int V,
-    int D, int blank, int ND, int Us, int A, int nchunks, int nblocks, GridDiv gdiv) {
+    int D, int nbig, int blank, int ND, int Us, int A, int nchunks, int nblocks, GridDiv gdiv) {
   constexpr int VEC = Elem<DT>::VEC;
   // all kernel arguments are fetched in one go, not one batch per use (the loads this kernel wants
   // on the scalar unit are written as such, so the asm's side effect costs nothing)
   asm volatile("" ::"s"((uintptr_t)acts), "s"((uintptr_t)labels), "s"((uintptr_t)act_lens), "s"((uintptr_t)label_lens),
-               "s"((uintptr_t)denom), "s"((uintptr_t)arcs), "s"(T), "s"(U), "s"(V), "s"(D), "s"(blank), "s"(ND), "s"(Us),
+               "s"((uintptr_t)denom), "s"((uintptr_t)arcs), "s"(T), "s"(U), "s"(V), "s"(D), "s"(nbig), "s"(blank), "s"(ND), "s"(Us),
                "s"(A), "s"(nchunks), "s"(nblocks), "s"(gdiv.chunks.mul), "s"(gdiv.chunks.shift), "s"(gdiv.T.mul),
                "s"(gdiv.T.shift));
   const int lane = threadIdx.x & 63;
@@ -1498,7 +1752,7 @@ __global__ __launch_bounds__(kRowThreads) void denom_rows_kernel(
     d.xe = Elem<DT>::load1(acts, e0 + (ve >= 0 ? ve : blank));
     d.xb = Elem<DT>::load1(acts, e0 + blank);
     d.xl = Elem<DT>::load1(acts, e0 + (lab >= 0 ? lab : blank));
-    d.xd = Elem<DT>::load1(acts, e0 + (lane < D ? V + lane : blank));
+    d.xd = Elem<DT>::load1(acts, e0 + (lane < D ? V + lane : (lane < nbig ? blank - 1 - lane : blank)));
   };
   auto reduce = [&](int uu, int lab, const Row& d) {
     const RowSplit<DT> sp(d.mis, V);
@@ -1542,6 +1796,7 @@ __global__ __launch_bounds__(kRowThreads) void denom_rows_kernel(
       const float dden = -dm - logf(ds);
       if (lane < D) arcs[base + (size_t)(2 + lane) * Us] = xd + dden;
     }
+    if (lane < nbig) arcs[base + (size_t)(2 + lane) * Us] = d.xd + dn;  // big-blank log-probs (multi-blank)
   };
 
   Row cur, nxt;
@@ -1730,14 +1985,14 @@ template <int DT, int RT, int NVT>
 __global__ __launch_bounds__(BlockRows<RT>::THREADS) void denom_block_kernel(
     const void* __restrict__ acts, const int64_t* __restrict__ labels, const int64_t* __restrict__ act_lens,
     const int64_t* __restrict__ label_lens, float* __restrict__ denom, float* __restrict__ arcs, int T, int U, int V,
-    int D, int blank, int ND, int Us, int A, int nchunks, int nblocks, GridDiv gdiv) {
+    int D, int nbig, int blank, int ND, int Us, int A, int nchunks, int nblocks, GridDiv gdiv) {
   constexpr int VEC = Elem<DT>::VEC;
   constexpr int ROWS = BlockRows<RT>::ROWS, WPR = BlockRows<RT>::WPR, WAVES = BlockRows<RT>::THREADS / 64;
   __shared__ float2 part[WAVES];
   // all kernel arguments are fetched in one go, not one batch per use (the loads this kernel wants
   // on the scalar unit are written as such, so the asm's side effect costs nothing)
   asm volatile("" ::"s"((uintptr_t)acts), "s"((uintptr_t)labels), "s"((uintptr_t)act_lens), "s"((uintptr_t)label_lens),
-               "s"((uintptr_t)denom), "s"((uintptr_t)arcs), "s"(T), "s"(U), "s"(V), "s"(D), "s"(blank), "s"(ND), "s"(Us),
+               "s"((uintptr_t)denom), "s"((uintptr_t)arcs), "s"(T), "s"(U), "s"(V), "s"(D), "s"(nbig), "s"(blank), "s"(ND), "s"(Us),
                "s"(A), "s"(nchunks), "s"(nblocks), "s"(gdiv.chunks.mul), "s"(gdiv.chunks.shift), "s"(gdiv.T.mul),
                "s"(gdiv.T.shift));
   const int lane = threadIdx.x & 63;
@@ -1780,7 +2035,7 @@ __global__ __launch_bounds__(BlockRows<RT>::THREADS) void denom_block_kernel(
       const float x1 = Elem<DT>::load1(acts, e0 + (ve >= 0 ? ve : blank));
       xb = Elem<DT>::load1(acts, e0 + blank);
       xl = Elem<DT>::load1(acts, e0 + (lab >= 0 ? lab : blank));
-      xd = Elem<DT>::load1(acts, e0 + (lane < D ? V + lane : blank));
+      xd = Elem<DT>::load1(acts, e0 + (lane < D ? V + lane : (lane < nbig ? blank - 1 - lane : blank)));
       xe = ve >= 0 ? x1 : kNegInf;
     }
     float x[NVT][VEC];
@@ -1831,6 +2086,7 @@ __global__ __launch_bounds__(BlockRows<RT>::THREADS) void denom_block_kernel(
     const float dden = -dm - logf(ds);
     if (lane < D) arcs[base + (size_t)(2 + lane) * Us] = xdm + dden;
   }
+  if (lane < nbig) arcs[base + (size_t)(2 + lane) * Us] = xd + dn;  // big-blank log-probs (multi-blank)
 }
 
 template <int DT, int RT, int NVT, bool FUSED>
@@ -2051,22 +2307,27 @@ struct Common {
   int dt;
   const int64_t *labels, *act_lens, *label_lens;
   int B, T, U, V, D, blank;
+  int nbig;  // multi-blank: number of big blanks (their logits sit at blank-1-i); D is 0 then
   char* ws;
   hipStream_t stream;
   Layout L;
 };
 
 int check_common(const void* acts, int dt, const int64_t* labels, const int64_t* act_lens, const int64_t* label_lens,
-                 int B, int T, int U, int V, int D, int blank, void* ws, size_t ws_bytes, void* stream, Common* c) {
+                 int B, int T, int U, int V, int D, int blank, void* ws, size_t ws_bytes, void* stream, Common* c,
+                 int nbig = 0) {
   if (!acts || !act_lens || !label_lens || !ws) return MI_TRANSDUCER_INVALID_VALUE;
   if (U > 1 && !labels) return MI_TRANSDUCER_INVALID_VALUE;
   if (dt != MI_DTYPE_F32 && dt != MI_DTYPE_BF16 && dt != MI_DTYPE_F16) return MI_TRANSDUCER_INVALID_VALUE;
   if (V <= 0 || blank < 0 || blank >= V) return MI_TRANSDUCER_INVALID_VALUE;
-  if (!make_layout(B, T, U, D, &c->L)) return MI_TRANSDUCER_INVALID_VALUE;
+  // multi-blank: the big blanks take the extra arc planes and coefficient slots that durations take for TDT
+  if (nbig < 0 || nbig > MI_TRANSDUCER_MAX_BIG_BLANKS || (nbig > 0 && (D != 0 || blank - nbig < 0)))
+    return MI_TRANSDUCER_INVALID_VALUE;
+  if (!make_layout(B, T, U, nbig ? nbig : D, &c->L)) return MI_TRANSDUCER_INVALID_VALUE;
   if (ws_bytes < c->L.total || ((uintptr_t)ws & 255)) return MI_TRANSDUCER_INVALID_VALUE;
   if ((long long)B * T > 65535LL * 8) return MI_TRANSDUCER_INVALID_VALUE;  // grid-size limit of the long-row kernels
   c->acts = acts; c->dt = dt; c->labels = labels; c->act_lens = act_lens; c->label_lens = label_lens;
-  c->B = B; c->T = T; c->U = U; c->V = V; c->D = D; c->blank = blank;
+  c->B = B; c->T = T; c->U = U; c->V = V; c->D = D; c->blank = blank; c->nbig = nbig;
   c->ws = (char*)ws; c->stream = (hipStream_t)stream;
   return MI_TRANSDUCER_SUCCESS;
 }
@@ -2200,7 +2461,7 @@ int run_denom(const Common& c) {
   ProfScope prof(MI_PROFILE_DENOM, c.stream);
 #define LAUNCH_DENOM_ROWS(DT, RR)                                                                                   \
   hipLaunchKernelGGL((denom_rows_kernel<DT, RR>), chunk_grid(c), dim3(kRowThreads), 0, c.stream, c.acts, c.labels,           \
-                     c.act_lens, c.label_lens, denom, arcs, c.T, c.U, c.V, c.D, c.blank, L.ND, L.Us, L.A, chunks_of(c), chunk_blocks(c), make_griddiv(chunks_of(c), c.T))
+                     c.act_lens, c.label_lens, denom, arcs, c.T, c.U, c.V, c.D, c.nbig, c.blank, L.ND, L.Us, L.A, chunks_of(c), chunk_blocks(c), make_griddiv(chunks_of(c), c.T))
 #define LAUNCH_DENOM(DT)                                                                                            \
   do {                                                                                                              \
     switch (R) {                                                                                                    \
@@ -2210,14 +2471,14 @@ int run_denom(const Common& c) {
       case 8: LAUNCH_DENOM_ROWS(DT, 8); break;                                                                      \
       default:                                                                                                      \
         hipLaunchKernelGGL(denom_gather_kernel<DT>, g.grid, dim3(256), 0, c.stream, c.acts, c.labels, c.act_lens,   \
-                           c.label_lens, denom, arcs, c.T, c.U, c.V, c.D, c.blank, L.ND, L.Us, L.A, g.BT,           \
+                           c.label_lens, denom, arcs, c.T, c.U, c.V, c.D, c.nbig, c.blank, L.ND, L.Us, L.A, g.BT,           \
                            g.bt_chunk);                                                                             \
     }                                                                                                               \
   } while (0)
   const BlockPlan bp = denom_block_plan(c);
 #define LAUNCH_DENOM_BLOCK(DT, RT_, NVT_)                                                                           \
   hipLaunchKernelGGL((denom_block_kernel<DT, RT_, NVT_>), plan_grid(c, bp), dim3(bp.threads()), 0, c.stream, c.acts, \
-                     c.labels, c.act_lens, c.label_lens, denom, arcs, c.T, c.U, c.V, c.D, c.blank, L.ND, L.Us, L.A,  \
+                     c.labels, c.act_lens, c.label_lens, denom, arcs, c.T, c.U, c.V, c.D, c.nbig, c.blank, L.ND, L.Us, L.A,  \
                      plan_chunks(c, bp), plan_blocks(c, bp), make_griddiv(plan_chunks(c, bp), c.T))
 #define DENOM_BLOCK_F32(RT_, NVT_) LAUNCH_DENOM_BLOCK(MI_DTYPE_F32, RT_, NVT_)
 #define DENOM_BLOCK_BF16(RT_, NVT_) LAUNCH_DENOM_BLOCK(MI_DTYPE_BF16, RT_, NVT_)
@@ -2423,10 +2684,85 @@ int run_tdt_cells(const Common& c, const ScaleArg& sc, float lambda, float clamp
 
 // ----------------------------------------------------------------------------------------
 // C ABI
+int make_mb_params(int NB, const int32_t* durations, float sigma, MbParams* p) {
+  if (NB < 0 || NB > MI_TRANSDUCER_MAX_BIG_BLANKS || (NB > 0 && !durations)) return MI_TRANSDUCER_INVALID_VALUE;
+  p->NB = NB;
+  p->sigma = sigma;
+  int longest = 1;
+  for (int i = 0; i < MI_TRANSDUCER_MAX_BIG_BLANKS; ++i) p->dur[i] = 0;
+  for (int i = 0; i < NB; ++i) {
+    if (durations[i] < 1 || durations[i] > MI_TRANSDUCER_MAX_BLANK_DURATION) return MI_TRANSDUCER_INVALID_VALUE;
+    p->dur[i] = durations[i];
+    longest = durations[i] > longest ? durations[i] : longest;
+  }
+  p->R = longest + 1;
+  return MI_TRANSDUCER_SUCCESS;
+}
+
+int run_multiblank_lattice(const Common& c, float* costs, float lambda, int with_betas, const MbParams& prm) {
+  const Layout& L = c.L;
+  const float* arcs = (const float*)(c.ws + L.off_arcs);
+  double* alphas = (double*)(c.ws + L.off_alphas);
+  double* betas = (double*)(c.ws + L.off_betas);
+  double* ll = (double*)(c.ws + L.off_ll);
+  const unsigned grid = (unsigned)(with_betas ? 2 * c.B : c.B);
+  const int nbc = prm.NB <= 1 ? 1 : (prm.NB <= 2 ? 2 : (prm.NB <= 4 ? 4 : 8));
+  const size_t lds = (size_t)prm.R * (2 + nbc) * L.Us * sizeof(double);  // the alpha ring is the larger one
+  if (lds > 160 * 1024) return MI_TRANSDUCER_INVALID_VALUE;
+  ProfScope prof(MI_PROFILE_LATTICE, c.stream);
+#define LAUNCH_MB(NN)                                                                                               \
+  do {                                                                                                              \
+    if (lds > 48 * 1024 &&                                                                                          \
+        hipFuncSetAttribute((const void*)multiblank_lattice_kernel<NN>, hipFuncAttributeMaxDynamicSharedMemorySize, \
+                            (int)lds) != hipSuccess)                                                                \
+      return MI_TRANSDUCER_LAUNCH_FAILURE;                                                                          \
+    hipLaunchKernelGGL(multiblank_lattice_kernel<NN>, dim3(grid), dim3(L.Us), lds, c.stream, arcs, alphas, betas,   \
+                       ll, costs, c.act_lens, c.label_lens, c.T, c.U, L.ND, L.Us, L.A, cost_scale_of(lambda),       \
+                       with_betas, prm);                                                                            \
+  } while (0)
+  switch (nbc) {
+    case 1: LAUNCH_MB(1); break;
+    case 2: LAUNCH_MB(2); break;
+    case 4: LAUNCH_MB(4); break;
+    default: LAUNCH_MB(8); break;
+  }
+#undef LAUNCH_MB
+  return launch_status();
+}
+
+int run_multiblank_cells(const Common& c, const ScaleArg& sc, float lambda, float clamp, const MbParams& prm) {
+  const Layout& L = c.L;
+  const long long cells = (long long)c.B * c.T * c.U;
+  const unsigned grid = (unsigned)((cells + 255) / 256);
+  ProfScope prof(MI_PROFILE_CELL, c.stream);
+  hipLaunchKernelGGL(multiblank_cell_kernel, dim3(grid), dim3(256), 0, c.stream, (const float*)(c.ws + L.off_denom),
+                     (const float*)(c.ws + L.off_arcs), (const double*)(c.ws + L.off_alphas),
+                     (const double*)(c.ws + L.off_betas), (const double*)(c.ws + L.off_ll), c.labels, c.act_lens,
+                     c.label_lens, sc.ptr, sc.stride, sc.mul, (float*)(c.ws + L.off_coef), c.T, c.U, c.V, c.blank, L.ND,
+                     L.Us, L.A, L.CS, lambda, clamp, cells, prm);
+  return launch_status();
+}
+
+int run_multiblank_fixup(const Common& c, void* grads, const MbParams& prm) {
+  if (prm.NB == 0) return MI_TRANSDUCER_SUCCESS;
+  const Layout& L = c.L;
+  const long long cells = (long long)c.B * c.T * c.U;
+  const unsigned grid = (unsigned)((cells * prm.NB + 255) / 256);
+  const float* coef = (const float*)(c.ws + L.off_coef);
+#define LAUNCH_FIX(DT)                                                                                             \
+  hipLaunchKernelGGL(multiblank_fixup_kernel<DT>, dim3(grid), dim3(256), 0, c.stream, grads, coef, c.V, c.blank,    \
+                     prm.NB, L.CS, cells)
+  if (c.dt == MI_DTYPE_F32) LAUNCH_FIX(MI_DTYPE_F32);
+  else if (c.dt == MI_DTYPE_BF16) LAUNCH_FIX(MI_DTYPE_BF16);
+  else LAUNCH_FIX(MI_DTYPE_F16);
+#undef LAUNCH_FIX
+  return launch_status();
+}
+
 // ----------------------------------------------------------------------------------------
 extern "C" {
 
-int mi_transducer_abi_version(void) { return 6; }
+int mi_transducer_abi_version(void) { return 7; }
 
 int mi_transducer_workspace_bytes(int B, int T, int U, int D, size_t* out_bytes) {
   Layout L;
@@ -2526,6 +2862,55 @@ int mi_tdt_loss(const void* acts, int act_dtype, const int64_t* labels, const in
   return mi_tdt_backward(acts, act_dtype, labels, act_lens, label_lens, grads, grad_scale, grad_scale_stride, grad_mul,
                          0, B, T, U, V, D, durations_host, blank, fastemit_lambda, clamp, sigma, use_plain_rnnt,
                          workspace, workspace_bytes, stream);
+}
+
+int mi_multiblank_forward(const void* acts, int act_dtype, const int64_t* labels, const int64_t* act_lens,
+                          const int64_t* label_lens, float* costs, int B, int T, int U, int V, int num_big_blanks,
+                          const int32_t* big_blank_durations_host, int blank, float fastemit_lambda, float sigma,
+                          int with_betas, void* workspace, size_t workspace_bytes, void* stream) {
+  Common c;
+  MbParams prm;
+  if (!costs) return MI_TRANSDUCER_INVALID_VALUE;
+  int st = make_mb_params(num_big_blanks, big_blank_durations_host, sigma, &prm);
+  if (st) return st;
+  st = check_common(acts, act_dtype, labels, act_lens, label_lens, B, T, U, V, 0, blank, workspace, workspace_bytes,
+                    stream, &c, num_big_blanks);
+  if (st) return st;
+  if ((st = run_denom(c))) return st;
+  return run_multiblank_lattice(c, costs, fastemit_lambda, with_betas, prm);
+}
+
+int mi_multiblank_backward(const void* acts, int act_dtype, const int64_t* labels, const int64_t* act_lens,
+                           const int64_t* label_lens, void* grads, const float* grad_scale, int grad_scale_stride,
+                           float grad_mul, int B, int T, int U, int V, int num_big_blanks,
+                           const int32_t* big_blank_durations_host, int blank, float fastemit_lambda, float clamp,
+                           float sigma, void* workspace, size_t workspace_bytes, void* stream) {
+  Common c;
+  MbParams prm;
+  if (!grads || clamp < 0.f || grad_scale_stride < 0) return MI_TRANSDUCER_INVALID_VALUE;
+  int st = make_mb_params(num_big_blanks, big_blank_durations_host, sigma, &prm);
+  if (st) return st;
+  st = check_common(acts, act_dtype, labels, act_lens, label_lens, B, T, U, V, 0, blank, workspace, workspace_bytes,
+                    stream, &c, num_big_blanks);
+  if (st) return st;
+  const ScaleArg sc = {grad_scale, grad_scale_stride, grad_mul};
+  if ((st = run_multiblank_cells(c, sc, fastemit_lambda, clamp, prm))) return st;
+  if ((st = run_grad_stream(c, grads, 0, false, sc, fastemit_lambda, clamp))) return st;
+  return run_multiblank_fixup(c, grads, prm);
+}
+
+int mi_multiblank_loss(const void* acts, int act_dtype, const int64_t* labels, const int64_t* act_lens,
+                       const int64_t* label_lens, float* costs, void* grads, const float* grad_scale,
+                       int grad_scale_stride, float grad_mul, int B, int T, int U, int V, int num_big_blanks,
+                       const int32_t* big_blank_durations_host, int blank, float fastemit_lambda, float clamp,
+                       float sigma, void* workspace, size_t workspace_bytes, void* stream) {
+  int st = mi_multiblank_forward(acts, act_dtype, labels, act_lens, label_lens, costs, B, T, U, V, num_big_blanks,
+                                 big_blank_durations_host, blank, fastemit_lambda, sigma, grads != nullptr, workspace,
+                                 workspace_bytes, stream);
+  if (st || !grads) return st;
+  return mi_multiblank_backward(acts, act_dtype, labels, act_lens, label_lens, grads, grad_scale, grad_scale_stride,
+                                grad_mul, B, T, U, V, num_big_blanks, big_blank_durations_host, blank, fastemit_lambda,
+                                clamp, sigma, workspace, workspace_bytes, stream);
 }
 
 int mi_transducer_export_lattice(const void* workspace, size_t workspace_bytes, const int64_t* act_lens,
@@ -2656,7 +3041,7 @@ int mi_transducer_describe_plan(int act_dtype, int B, int T, int U, int V, int D
   if (!out || out_bytes == 0 || V <= 0 || !make_layout(B, T, U, D, &c.L)) return MI_TRANSDUCER_INVALID_VALUE;
   if (act_dtype != MI_DTYPE_F32 && act_dtype != MI_DTYPE_BF16 && act_dtype != MI_DTYPE_F16)
     return MI_TRANSDUCER_INVALID_VALUE;
-  c.acts = nullptr; c.dt = act_dtype; c.B = B; c.T = T; c.U = U; c.V = V; c.D = D;
+  c.acts = nullptr; c.dt = act_dtype; c.B = B; c.T = T; c.U = U; c.V = V; c.D = D; c.nbig = 0;
   const char* dt = act_dtype == MI_DTYPE_F32 ? "f32" : (act_dtype == MI_DTYPE_BF16 ? "bf16" : "f16");
   char denom[96], lattice[96], cells[48], grad[112];
   const BlockPlan dp = denom_block_plan(c);

@@ -195,6 +195,40 @@ def tdt_backward(
     _native.check_status(status, "Could not calculate gradients")
 
 
+def multiblank_forward(
+    acts, labels, act_lens, label_lens, costs, blank, big_blank_durations, fastemit_lambda, sigma, with_betas, workspace
+):
+    _require_gpu(acts, "multiblank_forward")
+    B, T, U, V = acts.shape
+    keep, dur_ptr = _durations_array(big_blank_durations)
+    with torch.cuda.device(acts.device):
+        status = _native.lib().mi_multiblank_forward(
+            _ptr(acts), _dtype_code(acts), _labels_ptr(labels), _ptr(act_lens), _ptr(label_lens), _ptr(costs),
+            B, T, U, V, len(big_blank_durations), dur_ptr, int(blank), float(fastemit_lambda), float(sigma),
+            int(bool(with_betas)), _ptr(workspace), workspace.numel(), _stream(acts.device),
+        )  # fmt: skip
+    del keep
+    _native.check_status(status, "Could not calculate forward scores")
+
+
+def multiblank_backward(
+    acts, labels, act_lens, label_lens, grads, grad_scale, blank, big_blank_durations, fastemit_lambda, clamp, sigma,
+    workspace, grad_scale_stride=1, grad_mul=1.0,
+):  # fmt: skip
+    _require_gpu(acts, "multiblank_backward")
+    B, T, U, V = acts.shape
+    keep, dur_ptr = _durations_array(big_blank_durations)
+    with torch.cuda.device(acts.device):
+        status = _native.lib().mi_multiblank_backward(
+            _ptr(acts), _dtype_code(acts), _labels_ptr(labels), _ptr(act_lens), _ptr(label_lens), _ptr(grads),
+            _ptr(grad_scale), int(grad_scale_stride), float(grad_mul), B, T, U, V, len(big_blank_durations), dur_ptr,
+            int(blank), float(fastemit_lambda), float(clamp), float(sigma), _ptr(workspace), workspace.numel(),
+            _stream(acts.device),
+        )  # fmt: skip
+    del keep
+    _native.check_status(status, "Could not calculate gradients")
+
+
 def export_lattice(workspace, act_lens, label_lens, B, T, U, num_durations=0):
     """(denom, alphas, betas, ll_forward, ll_backward) as plain float32 tensors, for stage-level checks."""
     dev = workspace.device
@@ -251,6 +285,31 @@ def tdt_loss_gpu(
             _ptr(acts), _dtype_code(acts), _labels_ptr(labels), _ptr(input_lengths), _ptr(label_lengths), _ptr(costs),
             _ptr(grads), None, 0, 1.0, B, T, U, VD - D, D, dur_ptr, int(blank_label), float(fastemit_lambda),
             float(clamp), float(sigma), int(bool(use_plain_rnnt)), _ptr(workspace), workspace.numel(),
+            _stream(acts.device),
+        )  # fmt: skip
+    del keep
+    _native.check_status(status, "Could not calculate forward scores")
+    return True
+
+
+def multiblank_rnnt_loss_gpu(
+    acts, labels, input_lengths, label_lengths, costs, grads, blank_label, big_blank_durations, fastemit_lambda, clamp,
+    num_threads=0, sigma=0.0,
+):  # fmt: skip
+    """Multi-blank counterpart (rnnt.py:366-483): acts [B,T,U,V] with the big blanks at blank_label-1-i;
+    costs is float32 [B], grads (or None) has the shape and dtype of acts."""
+    del num_threads
+    _require_gpu(acts, "multiblank_rnnt_loss_gpu")
+    B, T, U, V = acts.shape
+    workspace = new_workspace(acts, len(big_blank_durations))
+    if costs.dtype != torch.float32:
+        raise TypeError("costs must be float32")
+    keep, dur_ptr = _durations_array(big_blank_durations)
+    with torch.cuda.device(acts.device):
+        status = _native.lib().mi_multiblank_loss(
+            _ptr(acts), _dtype_code(acts), _labels_ptr(labels), _ptr(input_lengths), _ptr(label_lengths), _ptr(costs),
+            _ptr(grads), None, 0, 1.0, B, T, U, V, len(big_blank_durations), dur_ptr, int(blank_label),
+            float(fastemit_lambda), float(clamp), float(sigma), _ptr(workspace), workspace.numel(),
             _stream(acts.device),
         )  # fmt: skip
     del keep

@@ -29,7 +29,10 @@ from torch.nn import Module
 
 from speech_amd.rnnt_loss import rnnt
 
-__all__ = ['RNNTLossNumba', 'TDTLossNumba', 'RNNTLossMI355X', 'TDTLossMI355X', 'certify_inputs']
+__all__ = [
+    'RNNTLossNumba', 'TDTLossNumba', 'MultiblankRNNTLossNumba', 'RNNTLossMI355X', 'TDTLossMI355X',
+    'MultiblankRNNTLossMI355X', 'certify_inputs',
+]  # fmt: skip
 
 
 # Optional (MI_TRANSDUCER_OVERLAP=1): when the gradient will be needed, forward allocates it and,
@@ -299,6 +302,53 @@ class _TDTNumba(Function):
         return grads, None, None, None, None, None, None, None, None, None, None
 
 
+class _MultiblankRNNTNumba(Function):
+    """Multi-blank transducer loss (arXiv:2211.03541); rnnt_pytorch.py:199-268."""
+
+    @staticmethod
+    def forward(
+        ctx, acts, labels, act_lens, label_lens, blank, big_blank_durations, reduction, fastemit_lambda, clamp, sigma
+    ):
+        _certify_static(acts, labels, act_lens, label_lens)
+        if clamp < 0:
+            raise ValueError("`clamp` must be 0.0 or positive float value.")
+        if not acts.is_cuda:
+            raise NotImplementedError()  # rnnt_pytorch.py:226-229
+        _check_same_device(acts, labels, act_lens, label_lens)
+        durations = [int(d) for d in big_blank_durations]
+        if blank - len(durations) < 0 or blank >= acts.shape[-1]:
+            raise ValueError("the big blanks sit at blank-1-i: blank must leave room for them below it")
+        pending = _PendingLengthCheck(acts, act_lens, label_lens)
+
+        need_grad = ctx.needs_input_grad[0]
+        batch = acts.size(0)
+        costs = torch.empty(batch, device=acts.device, dtype=torch.float32)
+        workspace = rnnt.new_workspace(acts, len(durations))
+        rnnt.multiblank_forward(
+            acts, labels, act_lens, label_lens, costs, blank, durations, fastemit_lambda, sigma, need_grad, workspace
+        )
+        pending.finish()
+
+        # the reference allocates these costs in the dtype of acts (rnnt_pytorch.py:232)
+        costs = _reduce_costs(costs, reduction, batch).to(acts.dtype)
+        if need_grad:
+            ctx.save_for_backward(acts, labels, act_lens, label_lens, workspace)
+            ctx.params = (blank, durations, reduction, fastemit_lambda, clamp, sigma)
+        return costs
+
+    @staticmethod
+    def backward(ctx, grad_output):
+        acts, labels, act_lens, label_lens, workspace = ctx.saved_tensors
+        blank, durations, reduction, fastemit_lambda, clamp, sigma = ctx.params
+        grads = torch.empty_like(acts)
+        scale, stride, mul = _grad_scale(grad_output, reduction, acts.size(0), acts.device)
+        rnnt.multiblank_backward(
+            acts, labels, act_lens, label_lens, grads, scale, blank, durations, fastemit_lambda, clamp, sigma,
+            workspace, stride, mul,
+        )  # fmt: skip
+        return grads, None, None, None, None, None, None, None, None, None
+
+
 class RNNTLossNumba(Module):
     """
     Parameters:
@@ -378,7 +428,54 @@ class TDTLossNumba(Module):
         )
 
 
+class MultiblankRNNTLossNumba(Module):
+    """
+    Parameters:
+        blank (int): standard blank label.
+        big_blank_durations: durations of the big blanks, e.g. [2, 4, 8]; big blank i is token blank-1-i.
+        reduction, fastemit_lambda, clamp: as RNNTLossNumba.
+        sigma: logit under-normalisation constant (recommended 0.05).
+    """
+
+    def __init__(
+        self,
+        blank,
+        big_blank_durations,
+        reduction='mean',
+        fastemit_lambda: float = 0.0,
+        clamp: float = -1,
+        sigma: float = 0.0,
+    ):
+        super().__init__()
+        self.blank = blank
+        self.big_blank_durations = big_blank_durations
+        self.fastemit_lambda = fastemit_lambda
+        self.clamp = float(clamp) if clamp > 0 else 0.0
+        self.reduction = reduction
+        self.loss = _MultiblankRNNTNumba.apply
+        self.sigma = sigma
+
+    def forward(self, acts, labels, act_lens, label_lens):
+        """
+        acts: [B, T, U, V] logits over the tokens, the big blanks and the standard blank
+        labels, act_lens, label_lens: as RNNTLossNumba
+        """
+        return self.loss(
+            acts,
+            labels,
+            act_lens,
+            label_lens,
+            self.blank,
+            self.big_blank_durations,
+            self.reduction,
+            self.fastemit_lambda,
+            self.clamp,
+            self.sigma,
+        )
+
+
 # names that say what they are; the *Numba names are kept so that code written
 # against the reference runs unchanged
 RNNTLossMI355X = RNNTLossNumba
 TDTLossMI355X = TDTLossNumba
+MultiblankRNNTLossMI355X = MultiblankRNNTLossNumba
