@@ -13,7 +13,7 @@ lengths), inputs already in HBM.  Prints ONE JSON line:
   kernels      mean duration of each pipeline kernel over the timed steps (ms)
   copy_probe   bandwidth a plain device copy reaches on this GPU (GB/s, read + write)
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload 0..4] [--no-cpu-baseline]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload 0..5] [--no-cpu-baseline]
 """
 
 import argparse
@@ -67,6 +67,9 @@ def cpu_baseline(cfg, acts, labels, act_lens, label_lens, n_utt):
     if cfg.D:
         oracle.tdt_loss(x, lab, al, ll, cfg.blank, cfg.durations, cfg.sigma, lam, clamp, dtype=np.float32,
                         num_threads=threads)  # fmt: skip
+    elif cfg.big_blank_durations:
+        oracle.multiblank_loss(x, lab, al, ll, cfg.blank, cfg.big_blank_durations, cfg.sigma, lam, clamp,
+                               dtype=np.float32, num_threads=threads)  # fmt: skip
     else:
         oracle.rnnt_cpu_path(x, lab, al, ll, cfg.blank, lam, clamp, dtype=np.float32, num_threads=threads)
     dt = time.perf_counter() - t0
@@ -88,7 +91,7 @@ def main():
 
     import torch
 
-    from speech_amd import RNNTLossNumba, TDTLossNumba, _native, synthetic
+    from speech_amd import MultiblankRNNTLossNumba, RNNTLossNumba, TDTLossNumba, _native, synthetic
 
     if not torch.cuda.is_available():
         print("bench.py: no GPU visible", file=sys.stderr)
@@ -102,6 +105,9 @@ def main():
     if cfg.D:
         loss = TDTLossNumba(blank=cfg.blank, durations=cfg.durations, reduction='none',
                             fastemit_lambda=cfg.fastemit_lambda, clamp=cfg.clamp, sigma=cfg.sigma)  # fmt: skip
+    elif cfg.big_blank_durations:
+        loss = MultiblankRNNTLossNumba(blank=cfg.blank, big_blank_durations=cfg.big_blank_durations, reduction='none',
+                                       fastemit_lambda=cfg.fastemit_lambda, clamp=cfg.clamp, sigma=cfg.sigma)  # fmt: skip
     else:
         loss = RNNTLossNumba(blank=cfg.blank, reduction='none', fastemit_lambda=cfg.fastemit_lambda, clamp=cfg.clamp)
     nbytes = synthetic.algorithmic_bytes(cfg, act_lens, label_lens)
@@ -159,7 +165,8 @@ def main():
     from speech_amd.rnnt_loss import rnnt, rnnt_pytorch
 
     plan = _native.describe_plan(rnnt._dtype_code(acts), cfg.B, cfg.T, cfg.U, cfg.V, cfg.D,
-                                 max(cfg.durations) if cfg.D else 0)  # fmt: skip
+                                 max(cfg.durations) if cfg.D else 0,
+                                 num_big_blanks=len(cfg.big_blank_durations))  # fmt: skip
 
     grad_ms, grad_n = kernels["gradient_pass"]
     grad_avg_s = grad_ms * 1e-3 / max(grad_n, 1)

@@ -85,8 +85,8 @@ _SIGNATURES = {
     "mi_transducer_profile_enable": [_c_int, ctypes.c_uint],
     "mi_transducer_profile_read": [_c_int, ctypes.POINTER(_c_float), ctypes.POINTER(_c_int)],
     "mi_transducer_profile_disable": [],
-    "mi_transducer_describe_plan": [_c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, ctypes.c_char_p,
-                                    _c_size_t],
+    "mi_transducer_describe_plan": [_c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int,
+                                    ctypes.c_char_p, _c_size_t],
     "mi_transducer_copy_probe": [_vp, _vp, _c_size_t, _vp],
 }  # fmt: skip
 
@@ -142,13 +142,14 @@ PROFILE_KERNELS = {
 }
 
 
-def describe_plan(dtype_code, B, T, U, V, D=0, max_duration=0, use_plain_rnnt=False):
-    """{'denominators': kernel, 'lattice': kernel, 'cells': kernel or '-', 'gradient': kernel} for a shape."""
+def describe_plan(dtype_code, B, T, U, V, D=0, max_duration=0, use_plain_rnnt=False, num_big_blanks=0):
+    """{'denominators': kernel, 'lattice': kernel, 'cells': kernel or '-', 'gradient': kernel} for a shape
+    (D > 0: TDT with that many durations; num_big_blanks > 0: multi-blank, V counting the big blanks)."""
     buf = ctypes.create_string_buffer(512)
     check_status(
         lib().mi_transducer_describe_plan(
             int(dtype_code), int(B), int(T), int(U), int(V), int(D), int(max_duration), int(bool(use_plain_rnnt)),
-            buf, ctypes.c_size_t(len(buf)),
+            int(num_big_blanks), buf, ctypes.c_size_t(len(buf)),
         ),
         "describe_plan",
     )

@@ -1273,8 +1273,10 @@ struct MbParams {
   float sigma;
 };
 
-template <int NBC>
-__global__ __launch_bounds__(1024) void multiblank_lattice_kernel(
+// MAXT: the largest workgroup the instantiation is launched with (256 leaves the compiler the whole
+// register file; the 1024-thread variant for U > 256 has to make do with 128 registers per thread)
+template <int NBC, int MAXT>
+__global__ __launch_bounds__(MAXT) void multiblank_lattice_kernel(
     const float* __restrict__ arcs, double* __restrict__ alphas, double* __restrict__ betas, double* __restrict__ ll,
     float* __restrict__ costs, const int64_t* __restrict__ act_lens, const int64_t* __restrict__ label_lens, int T,
     int U, int ND, int Us, int A, float cost_scale, int with_betas, MbParams prm) {
@@ -2710,15 +2712,19 @@ int run_multiblank_lattice(const Common& c, float* costs, float lambda, int with
   const size_t lds = (size_t)prm.R * (2 + nbc) * L.Us * sizeof(double);  // the alpha ring is the larger one
   if (lds > 160 * 1024) return MI_TRANSDUCER_INVALID_VALUE;
   ProfScope prof(MI_PROFILE_LATTICE, c.stream);
-#define LAUNCH_MB(NN)                                                                                               \
+#define LAUNCH_MB_T(NN, TT)                                                                                         \
   do {                                                                                                              \
-    if (lds > 48 * 1024 &&                                                                                          \
-        hipFuncSetAttribute((const void*)multiblank_lattice_kernel<NN>, hipFuncAttributeMaxDynamicSharedMemorySize, \
-                            (int)lds) != hipSuccess)                                                                \
+    if (lds > 48 * 1024 && hipFuncSetAttribute((const void*)multiblank_lattice_kernel<NN, TT>,                      \
+                                               hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) != hipSuccess) \
       return MI_TRANSDUCER_LAUNCH_FAILURE;                                                                          \
-    hipLaunchKernelGGL(multiblank_lattice_kernel<NN>, dim3(grid), dim3(L.Us), lds, c.stream, arcs, alphas, betas,   \
-                       ll, costs, c.act_lens, c.label_lens, c.T, c.U, L.ND, L.Us, L.A, cost_scale_of(lambda),       \
-                       with_betas, prm);                                                                            \
+    hipLaunchKernelGGL((multiblank_lattice_kernel<NN, TT>), dim3(grid), dim3(L.Us), lds, c.stream, arcs, alphas,    \
+                       betas, ll, costs, c.act_lens, c.label_lens, c.T, c.U, L.ND, L.Us, L.A,                       \
+                       cost_scale_of(lambda), with_betas, prm);                                                     \
+  } while (0)
+#define LAUNCH_MB(NN)                     \
+  do {                                    \
+    if (L.Us <= 256) LAUNCH_MB_T(NN, 256); \
+    else LAUNCH_MB_T(NN, 1024);           \
   } while (0)
   switch (nbc) {
     case 1: LAUNCH_MB(1); break;
@@ -2726,6 +2732,7 @@ int run_multiblank_lattice(const Common& c, float* costs, float lambda, int with
     case 4: LAUNCH_MB(4); break;
     default: LAUNCH_MB(8); break;
   }
+#undef LAUNCH_MB_T
 #undef LAUNCH_MB
   return launch_status();
 }
@@ -3036,9 +3043,11 @@ int mi_transducer_profile_disable(void) {
 }
 
 int mi_transducer_describe_plan(int act_dtype, int B, int T, int U, int V, int D, int max_duration,
-                                int use_plain_rnnt, char* out, size_t out_bytes) {
+                                int use_plain_rnnt, int num_big_blanks, char* out, size_t out_bytes) {
   Common c;
-  if (!out || out_bytes == 0 || V <= 0 || !make_layout(B, T, U, D, &c.L)) return MI_TRANSDUCER_INVALID_VALUE;
+  if (!out || out_bytes == 0 || V <= 0 || num_big_blanks < 0 || num_big_blanks > MI_TRANSDUCER_MAX_BIG_BLANKS ||
+      (num_big_blanks > 0 && D != 0) || !make_layout(B, T, U, num_big_blanks ? num_big_blanks : D, &c.L))
+    return MI_TRANSDUCER_INVALID_VALUE;
   if (act_dtype != MI_DTYPE_F32 && act_dtype != MI_DTYPE_BF16 && act_dtype != MI_DTYPE_F16)
     return MI_TRANSDUCER_INVALID_VALUE;
   c.acts = nullptr; c.dt = act_dtype; c.B = B; c.T = T; c.U = U; c.V = V; c.D = D; c.nbig = 0;
@@ -3049,7 +3058,11 @@ int mi_transducer_describe_plan(int act_dtype, int B, int T, int U, int V, int D
   else if (rows_R(c)) snprintf(denom, sizeof denom, "denom_rows_kernel<%s, R=%d>", dt, rows_R(c));
   else snprintf(denom, sizeof denom, "denom_gather_kernel<%s>", dt);
   const bool tdt = D > 0 && !use_plain_rnnt;
-  if (D == 0 || use_plain_rnnt) {
+  const bool mb = num_big_blanks > 0;
+  if (mb) {
+    const int nbc = num_big_blanks <= 1 ? 1 : (num_big_blanks <= 2 ? 2 : (num_big_blanks <= 4 ? 4 : 8));
+    snprintf(lattice, sizeof lattice, "multiblank_lattice_kernel<NBC=%d>", nbc);
+  } else if (D == 0 || use_plain_rnnt) {
     snprintf(lattice, sizeof lattice, "rnnt_lattice_kernel<K=%d>", c.L.K);
   } else {
     const int R = max_duration + 2;
@@ -3059,12 +3072,13 @@ int mi_transducer_describe_plan(int act_dtype, int B, int T, int U, int V, int D
   }
   // a gradient buffer at the 16-byte phase of the logits is assumed (what every allocator returns)
   const BlockPlan gp = grad_block_plan(c, nullptr);
-  const bool fused = !tdt && (gp.RT != 0 || rows_R(c) != 0);
-  snprintf(cells, sizeof cells, "%s", fused ? "-" : (tdt ? "tdt_cell_kernel" : "rnnt_cell_kernel"));
+  const bool fused = !tdt && !mb && (gp.RT != 0 || rows_R(c) != 0);
+  snprintf(cells, sizeof cells, "%s", fused ? "-" : (mb ? "multiblank_cell_kernel" : (tdt ? "tdt_cell_kernel" : "rnnt_cell_kernel")));
   if (gp.RT) snprintf(grad, sizeof grad, "grad_block_kernel<%s, RT=%d, NVT=%d, %s>", dt, gp.RT, gp.NVT, fused ? "fused" : "coef");
   else if (rows_R(c)) snprintf(grad, sizeof grad, "grad_rows_kernel<%s, R=%d, %s>", dt, rows_R(c), fused ? "fused" : "coef");
   else snprintf(grad, sizeof grad, "grad_stream_kernel<%s>", dt);
-  const int n = snprintf(out, out_bytes, "denominators=%s; lattice=%s; cells=%s; gradient=%s", denom, lattice, cells, grad);
+  const int n = snprintf(out, out_bytes, "denominators=%s; lattice=%s; cells=%s; gradient=%s%s", denom, lattice, cells,
+                         grad, mb ? " + multiblank_fixup_kernel" : "");
   return (n < 0 || (size_t)n >= out_bytes) ? MI_TRANSDUCER_INVALID_VALUE : MI_TRANSDUCER_SUCCESS;
 }
 

@@ -1,4 +1,5 @@
-"""Seeded synthetic inputs for the five benchmark configurations of the transducer loss.
+"""Seeded synthetic inputs for the five benchmark configurations of the transducer loss (plus one for the
+multi-blank loss, which the reference publishes no configuration for).
 
 Tensors are generated on the CPU with torch.Generator().manual_seed(1234 + index) so
 that the GPU path, the CPU baseline and the parity checks see identical values.
@@ -27,6 +28,8 @@ class Config:
     clamp: float = -1.0
     durations: List[int] = field(default_factory=list)
     sigma: float = 0.0
+    # multi-blank: durations of the big blanks; V then counts tokens + big blanks + the standard blank
+    big_blank_durations: List[int] = field(default_factory=list)
     zipf_labels: bool = False
 
     @property
@@ -51,6 +54,9 @@ CONFIGS = [
            durations=[0, 1, 2, 3, 4], sigma=0.05),
     Config("cfg5_rnnt_B8_T250_U101_V16385_f32", 8, 250, 101, 16385, t_min=150, u_min=30, fastemit_lambda=0.001,
            clamp=5.0, zipf_labels=True),
+    # the north-star shape with three big blanks appended to the vocabulary
+    Config("cfg6_multiblank_B16_T375_U121_V1028_f32", 16, 375, 121, 1028, t_min=200, u_min=40,
+           big_blank_durations=[2, 4, 8], sigma=0.05),
 ]  # fmt: skip
 
 
@@ -67,7 +73,7 @@ def make_lengths(cfg, gen):
 
 
 def make_labels(cfg, gen):
-    n_tokens = cfg.V - 1
+    n_tokens = cfg.V - 1 - len(cfg.big_blank_durations)
     if not cfg.zipf_labels:
         return torch.randint(0, n_tokens, (cfg.B, cfg.U - 1), generator=gen, dtype=torch.int64)
     # Zipf(s = 1.1) over [0, n_tokens) by inverse-CDF sampling of a seeded uniform

@@ -75,8 +75,13 @@ def test_kernel_plan_of_the_documented_shapes(built_lib):
     assert p["gradient"] == "grad_block_kernel<f32, RT=128, NVT=2, coef>"
     p = plan(F32, 16, 375, 121, 1025, D=5, max_duration=4, use_plain_rnnt=True)
     assert p["lattice"] == "rnnt_lattice_kernel<K=2>" and p["cells"] == "-"
+    p = plan(F32, 16, 375, 121, 1028, num_big_blanks=3)  # multi-blank: three big blanks inside V
+    assert p["lattice"] == "multiblank_lattice_kernel<NBC=4>" and p["cells"] == "multiblank_cell_kernel"
+    assert p["gradient"] == "grad_block_kernel<f32, RT=256, NVT=2, coef> + multiblank_fixup_kernel"
     with pytest.raises(RuntimeError):
         plan(7, 1, 1, 1, 5)
+    with pytest.raises(RuntimeError):
+        plan(F32, 1, 4, 2, 9, D=2, max_duration=1, num_big_blanks=2)  # TDT and multi-blank exclude each other
 
 
 def test_constructor_attributes_match_the_reference_conventions():
