@@ -20,8 +20,10 @@ What is done differently underneath:
     overlaps the forward kernels instead of two blocking torch.max calls.
 """
 
+import contextlib
 import os
 import random
+import threading
 
 import torch
 from torch.autograd import Function
@@ -83,12 +85,39 @@ def check_dim(var, dim, name):
         raise ValueError("{} must be {}D".format(name, dim))
 
 
+class _CallerMode(threading.local):
+    """How the next module call treats two things a wrapper around it decides (set only by
+    speech_amd.losses.rnnt.RNNTLoss, which stands where nemo/collections/asr/losses/rnnt.py:438-505 stands):
+    padded_time_axis  accept T >= max(act_lens): the wrapper of the reference trims the time axis with
+                      narrow().contiguous() before the call; the kernels skip padded frames anyway, so
+                      the copy is not made and the frames beyond max(act_lens) get a zero gradient
+    float32_costs     keep the costs in float32 whatever the dtype of acts (the reference's wrapper
+                      upcasts 16-bit logits before the call, so its costs are float32)"""
+
+    padded_time_axis = False
+    float32_costs = False
+
+
+_caller_mode = _CallerMode()
+
+
+@contextlib.contextmanager
+def wrapper_call_mode():
+    old = (_caller_mode.padded_time_axis, _caller_mode.float32_costs)
+    _caller_mode.padded_time_axis = _caller_mode.float32_costs = True
+    try:
+        yield
+    finally:
+        _caller_mode.padded_time_axis, _caller_mode.float32_costs = old
+
+
 class _PendingLengthCheck:
     """The T == max(act_lens), U == max(label_lens)+1 test of certify_inputs, split in two
     so that the read-back of the maxima overlaps kernels enqueued in between."""
 
     def __init__(self, log_probs, lengths, label_lengths):
         self.T, self.U = log_probs.shape[1:3]
+        self.padded_T = _caller_mode.padded_time_axis
         if lengths.is_cuda:
             # One small kernel on the auxiliary stream, ordered after whatever produced the lengths
             # on the current stream, writes the two maxima into pinned host memory: it runs beside
@@ -111,7 +140,7 @@ class _PendingLengthCheck:
         if self.event is not None:
             self.event.synchronize()
         max_T, max_U = int(self.host[0]), int(self.host[1])
-        if self.T != max_T:
+        if self.T < max_T if self.padded_T else self.T != max_T:
             raise ValueError(f"Input length mismatch! Given T: {self.T}, Expected max T from input lengths: {max_T}")
         if self.U != max_U + 1:
             raise ValueError(
@@ -280,7 +309,9 @@ class _TDTNumba(Function):
         pending.finish()
 
         # the reference allocates TDT costs in the dtype of acts (rnnt_pytorch.py:145)
-        costs = _reduce_costs(costs, reduction, batch).to(acts.dtype)
+        costs = _reduce_costs(costs, reduction, batch)
+        if not _caller_mode.float32_costs:
+            costs = costs.to(acts.dtype)
         if need_grad:
             ctx.save_for_backward(acts, labels, act_lens, label_lens, workspace)
             ctx.params = (blank, durations, reduction, fastemit_lambda, clamp, sigma, use_plain_rnnt)
@@ -330,7 +361,9 @@ class _MultiblankRNNTNumba(Function):
         pending.finish()
 
         # the reference allocates these costs in the dtype of acts (rnnt_pytorch.py:232)
-        costs = _reduce_costs(costs, reduction, batch).to(acts.dtype)
+        costs = _reduce_costs(costs, reduction, batch)
+        if not _caller_mode.float32_costs:
+            costs = costs.to(acts.dtype)
         if need_grad:
             ctx.save_for_backward(acts, labels, act_lens, label_lens, workspace)
             ctx.params = (blank, durations, reduction, fastemit_lambda, clamp, sigma)
