@@ -1266,6 +1266,14 @@ __global__ __launch_bounds__(256) void tdt_cell_kernel(
 // Cells outside the lattice hold "log 0" or junk that no valid cell reads, as in the RNNT kernel.
 // NBC is the compiled capacity for big blanks; prm.NB <= NBC are in use.
 // ----------------------------------------------------------------------------------------
+// Workgroup barrier that waits for this wave's LDS traffic only.  __syncthreads() also drains the
+// vector-memory counters: at every step of a recursion it would wait for the lattice store to be
+// acknowledged and for the prefetched arc rows to arrive.
+__device__ __forceinline__ void lds_barrier() {
+  __builtin_amdgcn_s_waitcnt(0xc07f);  // lgkmcnt(0); vmcnt and expcnt left alone
+  __builtin_amdgcn_s_barrier();
+}
+
 struct MbParams {
   int NB;
   int dur[MI_TRANSDUCER_MAX_BIG_BLANKS];
@@ -1296,6 +1304,16 @@ __global__ __launch_bounds__(MAXT) void multiblank_lattice_kernel(
   dur[0] = 1;
 #pragma unroll
   for (int j = 1; j < NJ; ++j) dur[j] = j - 1 < NB ? prm.dur[j - 1] : (1 << 28);  // unused slots never fire
+  // The step holds no test of NB (a wave-uniform test becomes a taken branch, and a lone wave per SIMD
+  // pays for every one of them): unused slots read an existing arc plane and their scores are pushed
+  // down to log 0 by this penalty.
+  double unused[NJ];
+  int plane[NJ];
+#pragma unroll
+  for (int j = 0; j < NJ; ++j) {
+    unused[j] = j - 1 < NB ? 0.0 : kLogZero;
+    plane[j] = j == 0 ? 0 : (j - 1 < NB ? 1 + j : 0);
+  }
   const size_t row_pitch = (size_t)A * Us;
   const float* arcs_b = arcs + (size_t)b * ND * row_pitch + u;
 
@@ -1309,7 +1327,7 @@ __global__ __launch_bounds__(MAXT) void multiblank_lattice_kernel(
       W[p][0] = finite_arc(rp[0]);
       W[p][1] = finite_arc(rp[Us]);
 #pragma unroll
-      for (int i = 0; i < NBC; ++i) W[p][2 + i] = i < NB ? finite_arc(rp[(size_t)(2 + i) * Us]) : 0.f;
+      for (int i = 0; i < NBC; ++i) W[p][2 + i] = finite_arc(rp[(size_t)plane[1 + i] * Us]);
     }
   };
   // log-sum-exp of x[0..N); "log 0" entries vanish, all "log 0" stays "log 0"
@@ -1353,13 +1371,13 @@ __global__ __launch_bounds__(MAXT) void multiblank_lattice_kernel(
 #pragma unroll
       for (int j = 0; j < NJ; ++j) {
         const double ob = (a + (double)w[j == 0 ? 0 : 1 + j]) - sigma;
-        slot[(1 + j) * Us] = j - 1 < NB ? ob : NINF;
-        final_arc[j] = (j - 1 < NB && u == Ub - 1 && t >= 0 && t + dur[j] == Tb) ? ob : final_arc[j];
+        slot[(1 + j) * Us] = ob + unused[j];
+        final_arc[j] = (u == Ub - 1 && t >= 0 && t + dur[j] == Tb) ? ob : final_arc[j];
       }
 #pragma unroll
       for (int j = 0; j < NJ; ++j) off_in[j] = off_in[j] + slot_stride == ring_len ? 0 : off_in[j] + slot_stride;
       cur_off = cur_off + slot_stride == ring_len ? 0 : cur_off + slot_stride;
-      __syncthreads();
+      lds_barrier();
     };
     float wa[P][2 + NBC], wb[P][2 + NBC];
     int n0 = 0;
@@ -1404,14 +1422,11 @@ __global__ __launch_bounds__(MAXT) void multiblank_lattice_kernel(
 #pragma unroll
       for (int j = 0; j < NJ; ++j) {
         const double arc = (double)w[j == 0 ? 0 : 1 + j] - sigma;
-        double xb = NINF;
-        if (j - 1 < NB) {
-          if (t + dur[j] < Tb) xb = ring[off_in[j] + u] + arc;
-          // a big blank may end the utterance from column Ub-1 (gpu_rnnt_kernel.py:660-670; the standard
-          // blank does so through the corner cell)
-          else if (j > 0 && t + dur[j] == Tb && u == Ub - 1 && dur[j] != 1) xb = arc;
-        }
-        x[1 + j] = xb;
+        // a big blank may end the utterance from column Ub-1 (gpu_rnnt_kernel.py:660-670; the standard
+        // blank does so through the corner cell); selects, not branches
+        const double via = ring[off_in[j] + u] + arc;
+        const bool ends = j > 0 && t + dur[j] == Tb && u == Ub - 1 && dur[j] != 1;
+        x[1 + j] = t + dur[j] < Tb ? via : (ends ? arc : NINF);
       }
       double v = lse_all(x);
       if (t == Tb - 1 && u == Ub - 1) v = (double)w[0] - sigma;  // the corner: one standard blank
@@ -1421,7 +1436,7 @@ __global__ __launch_bounds__(MAXT) void multiblank_lattice_kernel(
 #pragma unroll
       for (int j = 0; j < NJ; ++j) off_in[j] = off_in[j] == 0 ? ring_len - Us : off_in[j] - Us;
       cur_off = cur_off == 0 ? ring_len - Us : cur_off - Us;
-      __syncthreads();
+      lds_barrier();
     };
     float wa[P][2 + NBC], wb[P][2 + NBC];
     int n0 = nd - 1;
