@@ -850,9 +850,18 @@ __global__ __launch_bounds__(256) void tdt_lattice_block_kernel(
   const int R = prm.R;
   const double sigma = (double)prm.sigma;
   const double NEG = kTdtNeg;
-  int dur[D];
+  // dur_b: the duration as a BLANK arc sees it; a blank must advance, so duration 0 gets a value that
+  // never passes a time test.  The steps below are written with selects only: a wave-uniform test (on a
+  // duration, on the position of duration 1) would become a taken branch, and with one wave per SIMD
+  // every taken branch is paid in full.
+  int dur[D], dur_b[D];
 #pragma unroll
-  for (int i = 0; i < D; ++i) dur[i] = prm.dur[i];
+  for (int i = 0; i < D; ++i) {
+    dur[i] = prm.dur[i];
+    dur_b[i] = prm.dur[i] > 0 ? prm.dur[i] : (1 << 28);
+  }
+  const bool stay = prm.dur[0] == 0;  // a label may stay on its frame
+  const bool one_first = prm.one_idx == 0;
   const size_t row_pitch = (size_t)A * Us;
   const float* arcs_b = arcs + (size_t)b * ND * row_pitch + u;
 
@@ -904,15 +913,16 @@ __global__ __launch_bounds__(256) void tdt_lattice_block_kernel(
 #pragma unroll
       for (int i = 0; i < D; ++i) {
         const int d = dur[i];
-        const double vb = ring[off_b[i] + i * Us + u];
-        const double vl = ring[off_l[i] + (D + i) * Us + um1];
-        x[i] = (d > 0 && t >= d) ? vb : -INFINITY;
+        double vb = ring[off_b[i] + i * Us + u];
+        double vl = ring[off_l[i] + (D + i) * Us + um1];
+        asm("" : "+v"(vb), "+v"(vl));  // both reads are issued here, not under the tests that use them
+        x[i] = t >= dur_b[i] ? vb : -INFINITY;
         x[D + i] = (u > 0 && t >= d) ? vl : -INFINITY;
       }
-      double a;
-      if (t == 0 && u == 0) a = 0.0;
-      else if (t == 0) a = (dur[0] == 0) ? x[D] : NEG;  // only a duration-0 label arc reaches row 0 (:941-955)
-      else a = lse_all(x, u == 0 ? 1 : 2);              // the emit and the no-emit accumulator are both seeded
+      // the emit and the no-emit accumulator are both seeded; only a duration-0 label arc reaches row 0 (:941-955)
+      const double interior = lse_all(x, u == 0 ? 1 : 2);
+      const double row0 = u == 0 ? 0.0 : (stay ? x[D] : NEG);
+      const double a = t == 0 ? row0 : interior;
       out[(size_t)n * Us] = a;
       const double wb = a + (double)w[0], wl = a + (double)w[1];
       double* slot = ring + cur_off + u;
@@ -983,23 +993,19 @@ __global__ __launch_bounds__(256) void tdt_lattice_block_kernel(
         const int d = dur[i];
         const double dl = (double)w[2 + i];
         const double bw = (lpb + dl) - sigma, lw = (lpl + dl) - sigma;
-        const double vb = ring[off_b[i] + u];
-        const double vl = ring[off_l[i] + up1];
-        double xb = -INFINITY;
-        if (d > 0) {
-          if (t + d < Tb) xb = vb + bw;
-          else if (t + d == Tb && u == Ub - 1) xb = bw;
-        }
-        x[i] = xb;
+        double vb = ring[off_b[i] + u];
+        double vl = ring[off_l[i] + up1];
+        asm("" : "+v"(vb), "+v"(vl));  // both reads are issued here, not under the tests that use them
+        const int db = dur_b[i];
+        x[i] = t + db < Tb ? vb + bw : ((t + db == Tb && u == Ub - 1) ? bw : -INFINITY);
         x[D + i] = (t + d < Tb && u + 1 < Ub) ? vl + lw : -INFINITY;
       }
-      double v;
-      double corner = NEG;  // the corner ends the utterance with one blank of duration 1 (:1137-1148)
-#pragma unroll
-      for (int i = 0; i < D; ++i) corner = (i == prm.one_idx) ? x[i] : corner;
-      if (t == Tb - 1 && u == Ub - 1) v = corner;
-      else if (t == Tb - 1 && u < Ub - 1) v = (dur[0] == 0) ? x[D] : NEG;  // last row: duration-0 labels only
-      else v = lse_all(x, u == Ub - 1 ? 1 : 2);
+      // the corner ends the utterance with one blank of duration 1 (:1137-1148); the rest of the last row
+      // takes duration-0 labels only
+      const double corner = one_first ? x[0] : x[D > 1 ? 1 : 0];
+      const double interior = lse_all(x, u == Ub - 1 ? 1 : 2);
+      const double last_row = u == Ub - 1 ? corner : (stay ? x[D] : NEG);
+      const double v = t == Tb - 1 ? last_row : interior;
       out[(size_t)n * Us] = v;
       ring[cur_off + u] = v;
       last = v;
