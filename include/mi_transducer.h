@@ -198,7 +198,7 @@ int mi_transducer_length_maxima(const int64_t* act_lens, const int64_t* label_le
  * launches of one kernel class, returns their summed duration and count, and resets that
  * class.  Not thread-safe; leave disabled outside benchmarks. */
 #define MI_PROFILE_DENOM 0   /* denom_rows_kernel / denom_block_kernel / denom_gather_kernel */
-#define MI_PROFILE_LATTICE 1 /* rnnt_lattice_kernel / tdt_lattice_block_kernel / tdt_lattice_kernel */
+#define MI_PROFILE_LATTICE 1 /* rnnt_lattice_kernel / tdt_lattice_pair_kernel / tdt_lattice_kernel */
 #define MI_PROFILE_CELL 2    /* rnnt_cell_kernel / tdt_cell_kernel */
 #define MI_PROFILE_GRAD 3    /* grad_rows_kernel / grad_block_kernel / grad_stream_kernel */
 #define MI_PROFILE_ZERO 4    /* zero_padding_kernel */

@@ -825,16 +825,20 @@ __global__ __launch_bounds__(64) void tdt_lattice_kernel(const float* __restrict
 }
 
 // TDT lattice, workgroup version (gpu_rnnt_kernel.py:888-1241): one workgroup per (utterance,
-// direction), one thread per column u, one anti-diagonal per step, one barrier per step.
+// direction), TWO threads per column u, one anti-diagonal per step, one barrier per step.
 //   alpha: a finished cell leaves its 2D outgoing arc scores (alpha + arc weight, blank arcs
 //          and label arcs per duration) in an LDS ring of R = max_duration + 2 diagonals; a
-//          cell's alpha is ONE log-sum-exp over the up to 2D-1 scores that land on it (max,
-//          sum of exp2 in fp32, one log), plus the reference's finite -10000 seeds.
-//   beta : the ring holds beta of the last R diagonals; arc weights are the cell's own.
-// The cell's arc weights (blank, label, D duration log-probs) do not depend on the recursion
-// and are fetched P diagonals ahead.
+//          cell's alpha is one log-sum-exp over the <= 2D scores that land on it plus the
+//          reference's finite -10000 seeds.
+//   beta : the ring holds beta of the last R diagonals.
+// Thread (u, 0) sums the D blank arcs of a cell, thread (u, 1) the D label arcs, and the two partial
+// (max, sum) pairs meet through one DPP exchange: the recursion is bound by the instructions one
+// wave has to issue per step, and this halves them (at twice the waves, which sit on other SIMDs).
+// The steps are written with selects only: a wave-uniform test (on a duration, on the position of
+// duration 1) would become a taken branch, and with one wave per SIMD every taken branch is paid in
+// full (measured: 392 us with such branches, 323 us without, 293 us with two threads per column).
 template <int D>
-__global__ __launch_bounds__(256) void tdt_lattice_block_kernel(
+__global__ __launch_bounds__(512) void tdt_lattice_pair_kernel(
     const float* __restrict__ arcs, double* __restrict__ alphas, double* __restrict__ betas, double* __restrict__ ll,
     float* __restrict__ costs, const int64_t* __restrict__ act_lens, const int64_t* __restrict__ label_lens, int T,
     int U, int ND, int Us, float cost_scale, int with_betas, TdtParams prm) {
@@ -843,106 +847,111 @@ __global__ __launch_bounds__(256) void tdt_lattice_block_kernel(
   extern __shared__ double ring[];
   const int b = with_betas ? (int)(blockIdx.x >> 1) : (int)blockIdx.x;
   const int dir = with_betas ? (int)(blockIdx.x & 1) : 0;
-  const int u = threadIdx.x;  // blockDim.x == Us
+  const int u = threadIdx.x >> 1;     // blockDim.x == 2 * Us
+  const bool lab = threadIdx.x & 1;   // this thread's half: label arcs (else blank arcs)
   const int Tb = clampi(act_lens[b], 1, T);
   const int Ub = clampi(label_lens[b] + 1, 1, U);
   const int nd = Tb + Ub - 1;
   const int R = prm.R;
   const double sigma = (double)prm.sigma;
   const double NEG = kTdtNeg;
-  // dur_b: the duration as a BLANK arc sees it; a blank must advance, so duration 0 gets a value that
-  // never passes a time test.  The steps below are written with selects only: a wave-uniform test (on a
-  // duration, on the position of duration 1) would become a taken branch, and with one wave per SIMD
-  // every taken branch is paid in full.
-  int dur[D], dur_b[D];
+  // thr: from which t (alpha) an arc of duration i exists for this half; a blank must advance, so its
+  // duration 0 never passes
+  int dur[D], thr[D];
 #pragma unroll
   for (int i = 0; i < D; ++i) {
     dur[i] = prm.dur[i];
-    dur_b[i] = prm.dur[i] > 0 ? prm.dur[i] : (1 << 28);
+    thr[i] = (lab || prm.dur[i] > 0) ? prm.dur[i] : (1 << 28);
   }
   const bool stay = prm.dur[0] == 0;  // a label may stay on its frame
   const bool one_first = prm.one_idx == 0;
   const size_t row_pitch = (size_t)A * Us;
   const float* arcs_b = arcs + (size_t)b * ND * row_pitch + u;
+  const int own_plane = lab ? 1 : 0;  // the token arc of this half: label or blank
 
-  auto load_rows = [&](int nfirst, int step, float(&W)[P][A]) {
+  // [0]: this half's token log-prob, [1+i]: duration log-probs
+  auto load_rows = [&](int nfirst, int step, float(&W)[P][1 + D]) {
 #pragma unroll
     for (int p = 0; p < P; ++p) {
       int n = nfirst + step * p;
       n = n < 0 ? 0 : (n >= nd ? nd - 1 : n);
       const float* rp = arcs_b + (size_t)n * row_pitch;
+      W[p][0] = rp[(size_t)own_plane * Us];
 #pragma unroll
-      for (int a = 0; a < A; ++a) W[p][a] = rp[(size_t)a * Us];
+      for (int i = 0; i < D; ++i) W[p][1 + i] = rp[(size_t)(2 + i) * Us];
     }
   };
-  // log-sum-exp of x[0..N) (entries may be -inf = absent) and `seeds` copies of the sentinel
-  auto lse_all = [&](const double* x, int seeds) {
-    double m = seeds > 0 ? NEG : -INFINITY;
+  // the other half's value (lanes 2k and 2k+1 swap)
+  auto partner_f = [&](float v) {
+    return __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0xB1, 0xf, 0xf, true));
+  };
+  auto partner_d = [&](double v) {
+    return __hiloint2double(__builtin_amdgcn_update_dpp(0, __double2hiint(v), 0xB1, 0xf, 0xf, true),
+                            __builtin_amdgcn_update_dpp(0, __double2loint(v), 0xB1, 0xf, 0xf, true));
+  };
+  // log-sum-exp over both halves: each half holds D entries (-inf = absent) and `seed` copies (0 or 1) of the sentinel
+  auto lse_pair = [&](const double* x, int seed) {
+    double m = seed > 0 ? NEG : -1.0e300;
 #pragma unroll
-    for (int i = 0; i < 2 * D; ++i) m = fmax(m, x[i]);
-    float s = (float)seeds * fast_exp2((float)(NEG - m) * kLog2e);
+    for (int i = 0; i < D; ++i) m = fmax(m, x[i]);
+    float s = seed > 0 ? fast_exp2((float)(NEG - m) * kLog2e) : 0.f;  // (not seed * exp: 0 * inf for an empty half)
 #pragma unroll
-    for (int i = 0; i < 2 * D; ++i) s += fast_exp2((float)(x[i] - m) * kLog2e);
-    return m + (double)(__builtin_amdgcn_logf(s) * 0.6931471805599453f);
+    for (int i = 0; i < D; ++i) s += fast_exp2((float)(x[i] - m) * kLog2e);
+    const double mo = partner_d(m);
+    const float so = partner_f(s);
+    const double M = fmax(m, mo);
+    const float S = s * fast_exp2((float)(m - M) * kLog2e) + so * fast_exp2((float)(mo - M) * kLog2e);
+    return M + (double)(__builtin_amdgcn_logf(S) * 0.6931471805599453f);
   };
 
   if (dir == 0) {
-    for (int i = u; i < R * 2 * D * Us; i += Us) ring[i] = NEG;
+    const int slot_stride = 2 * D * Us, ring_len = R * slot_stride;
+    for (int i = threadIdx.x; i < ring_len; i += 2 * Us) ring[i] = NEG;
     __syncthreads();
     double* out = alphas + (size_t)b * ND * Us + u;
-    // Ring offsets (in doubles) of the diagonals n - d_i, kept incrementally: R is a run-time value
-    // and the loop should hold no division.  The diagonal n-1-d_i of this step is the diagonal
-    // n-d_i of the previous step.
-    const int slot_stride = 2 * D * Us, ring_len = R * slot_stride;
-    int off_b[D], off_l[D];
+    // ring offsets of the diagonals this half reads: n - d_i (blank arcs, same column) or n - 1 - d_i
+    // (label arcs, column u-1); both advance by one slot per step
+    int off[D];
 #pragma unroll
-    for (int i = 0; i < D; ++i) {
-      off_b[i] = ((R - dur[i]) % R) * slot_stride;
-      off_l[i] = (R - 1 - dur[i]) * slot_stride;
-    }
-    int cur_off = 0;  // offset of diagonal n's own slot
-    const int um1 = u > 0 ? u - 1 : 0;
-    // the arcs that end the utterance (t + d_i == Tb at column Ub-1, :1040-1071) are kept as they
-    // pass and summed after the loop, in the order of their steps
+    for (int i = 0; i < D; ++i) off[i] = (lab ? (R - 1 - dur[i]) : ((R - dur[i]) % R)) * slot_stride;
+    int cur_off = 0;
+    const int col = lab ? (u > 0 ? u - 1 : 0) : u;
+    const int plane0 = lab ? D * Us : 0;
+    const bool half_on = !lab || u > 0;  // column 0 has no label arc coming in
+    const int seed = half_on ? 1 : 0;    // the emit and the no-emit accumulator are each seeded once
     double final_arc[D];
 #pragma unroll
     for (int i = 0; i < D; ++i) final_arc[i] = -INFINITY;
     auto step_fn = [&](int n, const float* w) {
       const int t = n - u;
-      double x[2 * D];
+      double x[D];
 #pragma unroll
       for (int i = 0; i < D; ++i) {
-        const int d = dur[i];
-        double vb = ring[off_b[i] + i * Us + u];
-        double vl = ring[off_l[i] + (D + i) * Us + um1];
-        asm("" : "+v"(vb), "+v"(vl));  // both reads are issued here, not under the tests that use them
-        x[i] = t >= dur_b[i] ? vb : -INFINITY;
-        x[D + i] = (u > 0 && t >= d) ? vl : -INFINITY;
+        double v = ring[off[i] + plane0 + i * Us + col];
+        asm("" : "+v"(v));  // read here, not under the test below
+        x[i] = (half_on && t >= thr[i]) ? v : -INFINITY;
       }
-      // the emit and the no-emit accumulator are both seeded; only a duration-0 label arc reaches row 0 (:941-955)
-      const double interior = lse_all(x, u == 0 ? 1 : 2);
-      const double row0 = u == 0 ? 0.0 : (stay ? x[D] : NEG);
+      const double interior = lse_pair(x, seed);
+      // row 0: only a duration-0 label arc gets there (:941-955); its score sits in the label half
+      const double x0_other = partner_d(x[0]);
+      const double label0 = lab ? x[0] : x0_other;
+      const double row0 = u == 0 ? 0.0 : (stay ? label0 : NEG);
       const double a = t == 0 ? row0 : interior;
-      out[(size_t)n * Us] = a;
-      const double wb = a + (double)w[0], wl = a + (double)w[1];
-      double* slot = ring + cur_off + u;
+      if (!lab) out[(size_t)n * Us] = a;
+      const double wt = (a + (double)w[0]) - sigma;
+      double* slot = ring + cur_off + plane0 + u;
 #pragma unroll
       for (int i = 0; i < D; ++i) {
-        const double dl = (double)w[2 + i];
-        const double ob = (wb - sigma) + dl;
+        const double ob = wt + (double)w[1 + i];
         slot[i * Us] = ob;
-        slot[(D + i) * Us] = (wl - sigma) + dl;
-        final_arc[i] = (dur[i] > 0 && u == Ub - 1 && t >= 0 && t + dur[i] == Tb) ? ob : final_arc[i];
+        final_arc[i] = (!lab && dur[i] > 0 && u == Ub - 1 && t >= 0 && t + dur[i] == Tb) ? ob : final_arc[i];  // :1040-1071
       }
 #pragma unroll
-      for (int i = 0; i < D; ++i) {
-        off_l[i] = off_b[i];
-        off_b[i] = off_b[i] + slot_stride == ring_len ? 0 : off_b[i] + slot_stride;
-      }
+      for (int i = 0; i < D; ++i) off[i] = off[i] + slot_stride == ring_len ? 0 : off[i] + slot_stride;
       cur_off = cur_off + slot_stride == ring_len ? 0 : cur_off + slot_stride;
       __syncthreads();
     };
-    float wa[P][A], wb[P][A];
+    float wa[P][1 + D], wb[P][1 + D];
     int n0 = 0;
     load_rows(0, 1, wa);
     for (; n0 + 2 * P <= nd; n0 += 2 * P) {
@@ -954,13 +963,12 @@ __global__ __launch_bounds__(256) void tdt_lattice_block_kernel(
       for (int p = 0; p < P; ++p) step_fn(n0 + P + p, wb[p]);
     }
     for (; n0 < nd; ++n0) {
-      float w[A];
-#pragma unroll
-      for (int a = 0; a < A; ++a) w[a] = arcs_b[(size_t)n0 * row_pitch + (size_t)a * Us];
-      step_fn(n0, w);
+      float w[P][1 + D];
+      load_rows(n0, 0, w);
+      step_fn(n0, w[0]);
     }
-    if (u == Ub - 1) {
-      // a longer duration ends the utterance from an earlier diagonal: that order, as in the loop
+    if (!lab && u == Ub - 1) {
+      // a longer duration ends the utterance from an earlier diagonal: summed in that order
       double ll_acc = NEG;
 #pragma unroll
       for (int i = D - 1; i >= 0; --i)
@@ -969,55 +977,52 @@ __global__ __launch_bounds__(256) void tdt_lattice_block_kernel(
       costs[b] = -(float)ll_acc * cost_scale;
     }
   } else {
-    for (int i = u; i < R * Us; i += Us) ring[i] = NEG;
+    const int ring_len = R * Us;
+    for (int i = threadIdx.x; i < ring_len; i += 2 * Us) ring[i] = NEG;
     __syncthreads();
     double* out = betas + (size_t)b * ND * Us + u;
     double last = NEG;
-    // ring offsets of the diagonals n + d_i; the diagonal n+d_i+1 of this step is the diagonal
-    // n+d_i of the previous step (n runs downwards)
-    const int ring_len = R * Us;
-    int off_b[D], off_l[D];
+    // ring offsets of the diagonals this half reads: n + d_i (blank arcs, same column) or n + d_i + 1
+    // (label arcs, column u+1); both go back by one slot per step
+    int off[D];
 #pragma unroll
-    for (int i = 0; i < D; ++i) {
-      off_b[i] = (((nd - 1) % R + dur[i]) % R) * Us;
-      off_l[i] = (((nd - 1) % R + dur[i] + 1) % R) * Us;
-    }
+    for (int i = 0; i < D; ++i) off[i] = (((nd - 1) % R + dur[i] + (lab ? 1 : 0)) % R) * Us;
     int cur_off = ((nd - 1) % R) * Us;
-    const int up1 = u + 1 < Us ? u + 1 : u;
+    const int col = lab ? (u + 1 < Us ? u + 1 : u) : u;
     auto step_fn = [&](int n, const float* w) {
       const int t = n - u;
-      const double lpb = (double)w[0], lpl = (double)w[1];
-      double x[2 * D];
+      const double tok = (double)w[0];
+      double x[D];
 #pragma unroll
       for (int i = 0; i < D; ++i) {
-        const int d = dur[i];
-        const double dl = (double)w[2 + i];
-        const double bw = (lpb + dl) - sigma, lw = (lpl + dl) - sigma;
-        double vb = ring[off_b[i] + u];
-        double vl = ring[off_l[i] + up1];
-        asm("" : "+v"(vb), "+v"(vl));  // both reads are issued here, not under the tests that use them
-        const int db = dur_b[i];
-        x[i] = t + db < Tb ? vb + bw : ((t + db == Tb && u == Ub - 1) ? bw : -INFINITY);
-        x[D + i] = (t + d < Tb && u + 1 < Ub) ? vl + lw : -INFINITY;
+        double v = ring[off[i] + col];
+        asm("" : "+v"(v));
+        const double arc = (tok + (double)w[1 + i]) - sigma;
+        const int d = thr[i];  // blank half: duration 0 never passes
+        const bool reach = t + d < Tb && (!lab || u + 1 < Ub);
+        const bool ends = !lab && t + d == Tb && u == Ub - 1;  // a blank that ends the utterance
+        x[i] = reach ? v + arc : (ends ? arc : -INFINITY);
       }
+      // one seed for the no-emit (blank) accumulator, one for the emit accumulator unless it is the last column
+      const double interior = lse_pair(x, (!lab || u != Ub - 1) ? 1 : 0);
       // the corner ends the utterance with one blank of duration 1 (:1137-1148); the rest of the last row
-      // takes duration-0 labels only
-      const double corner = one_first ? x[0] : x[D > 1 ? 1 : 0];
-      const double interior = lse_all(x, u == Ub - 1 ? 1 : 2);
-      const double last_row = u == Ub - 1 ? corner : (stay ? x[D] : NEG);
+      // takes duration-0 labels only.  Each half sends the partner the one value it may need.
+      const double send = lab ? x[0] : (one_first ? x[0] : x[D > 1 ? 1 : 0]);
+      const double recv = partner_d(send);
+      const double corner = lab ? recv : send, label0 = lab ? send : recv;
+      const double last_row = u == Ub - 1 ? corner : (stay ? label0 : NEG);
       const double v = t == Tb - 1 ? last_row : interior;
-      out[(size_t)n * Us] = v;
-      ring[cur_off + u] = v;
+      if (!lab) {
+        out[(size_t)n * Us] = v;
+        ring[cur_off + u] = v;
+      }
       last = v;
 #pragma unroll
-      for (int i = 0; i < D; ++i) {
-        off_l[i] = off_b[i];
-        off_b[i] = off_b[i] == 0 ? ring_len - Us : off_b[i] - Us;
-      }
+      for (int i = 0; i < D; ++i) off[i] = off[i] == 0 ? ring_len - Us : off[i] - Us;
       cur_off = cur_off == 0 ? ring_len - Us : cur_off - Us;
       __syncthreads();
     };
-    float wa[P][A], wb[P][A];
+    float wa[P][1 + D], wb[P][1 + D];
     int n0 = nd - 1;
     load_rows(n0, -1, wa);
     for (; n0 - 2 * P + 1 >= 0; n0 -= 2 * P) {
@@ -1029,12 +1034,11 @@ __global__ __launch_bounds__(256) void tdt_lattice_block_kernel(
       for (int p = 0; p < P; ++p) step_fn(n0 - P - p, wb[p]);
     }
     for (; n0 >= 0; --n0) {
-      float w[A];
-#pragma unroll
-      for (int a = 0; a < A; ++a) w[a] = arcs_b[(size_t)n0 * row_pitch + (size_t)a * Us];
-      step_fn(n0, w);
+      float w[P][1 + D];
+      load_rows(n0, 0, w);
+      step_fn(n0, w[0]);
     }
-    if (u == 0) ll[2 * b + 1] = last;  // beta(0,0)
+    if (threadIdx.x == 0) ll[2 * b + 1] = last;  // beta(0,0)
   }
 }
 
@@ -2560,10 +2564,10 @@ int run_tdt_lattice(const Common& c, float* costs, float lambda, int with_betas,
   if (prm.D <= 8 && L.Us <= 256 && lds_block <= 160 * 1024) {
 #define LAUNCH_TBLK(DD)                                                                                              \
   if (lds_block > 48 * 1024 &&                                                                                       \
-      hipFuncSetAttribute((const void*)tdt_lattice_block_kernel<DD>, hipFuncAttributeMaxDynamicSharedMemorySize,     \
+      hipFuncSetAttribute((const void*)tdt_lattice_pair_kernel<DD>, hipFuncAttributeMaxDynamicSharedMemorySize,      \
                           (int)lds_block) != hipSuccess)                                                             \
     return MI_TRANSDUCER_LAUNCH_FAILURE;                                                                             \
-  hipLaunchKernelGGL(tdt_lattice_block_kernel<DD>, dim3(grid), dim3(L.Us), lds_block, c.stream, arcs, alphas, betas,  \
+  hipLaunchKernelGGL(tdt_lattice_pair_kernel<DD>, dim3(grid), dim3(2 * L.Us), lds_block, c.stream, arcs, alphas, betas,  \
                      ll, costs, c.act_lens, c.label_lens, c.T, c.U, L.ND, L.Us, cost_scale_of(lambda), with_betas,   \
                      prm)
     switch (prm.D) {
@@ -3088,7 +3092,7 @@ int mi_transducer_describe_plan(int act_dtype, int B, int T, int U, int V, int D
   } else {
     const int R = max_duration + 2;
     const size_t lds_block = (size_t)R * 2 * D * c.L.Us * sizeof(double);
-    if (D <= 8 && c.L.Us <= 256 && lds_block <= 160 * 1024) snprintf(lattice, sizeof lattice, "tdt_lattice_block_kernel<D=%d>", D);
+    if (D <= 8 && c.L.Us <= 256 && lds_block <= 160 * 1024) snprintf(lattice, sizeof lattice, "tdt_lattice_pair_kernel<D=%d>", D);
     else snprintf(lattice, sizeof lattice, "tdt_lattice_kernel<K=%d>", c.L.K);
   }
   // a gradient buffer at the 16-byte phase of the logits is assumed (what every allocator returns)

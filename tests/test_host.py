@@ -71,7 +71,7 @@ def test_kernel_plan_of_the_documented_shapes(built_lib):
     assert p["denominators"] == "denom_gather_kernel<f32>" and p["gradient"] == "grad_stream_kernel<f32>"
     assert p["cells"] == "rnnt_cell_kernel"
     p = plan(F32, 16, 375, 121, 1025, D=5, max_duration=4)  # TDT: coefficients come from the cell kernel
-    assert p["lattice"] == "tdt_lattice_block_kernel<D=5>" and p["cells"] == "tdt_cell_kernel"
+    assert p["lattice"] == "tdt_lattice_pair_kernel<D=5>" and p["cells"] == "tdt_cell_kernel"
     assert p["gradient"] == "grad_block_kernel<f32, RT=128, NVT=2, coef>"
     p = plan(F32, 16, 375, 121, 1025, D=5, max_duration=4, use_plain_rnnt=True)
     assert p["lattice"] == "rnnt_lattice_kernel<K=2>" and p["cells"] == "-"
