@@ -112,11 +112,8 @@ __device__ __forceinline__ float wave_sum(float v) {
 }
 
 __device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
-#ifdef MI_EXPERIMENT_NO_EXP
-__device__ __forceinline__ float stream_exp2(float x) { return x * 1e-3f; }
-#else
+// the exponential of the two streaming passes (one hardware v_exp_f32 per logit)
 __device__ __forceinline__ float stream_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
-#endif
 __device__ __forceinline__ float clamp_sym(float g, float bound) { return fminf(fmaxf(g, -bound), bound); }
 
 // Element access for the three logit dtypes.  A "vector" is 16 bytes.
@@ -1184,18 +1181,19 @@ __device__ __forceinline__ RowCoef finish_coef(const CoefRaw& r, const LatticeVi
                    scale);
 }
 
-__global__ __launch_bounds__(256) void rnnt_cell_kernel(
+__global__ __launch_bounds__(1024) void rnnt_cell_kernel(
     const float* __restrict__ denom, const float* __restrict__ arcs, const double* __restrict__ alphas,
     const double* __restrict__ betas, const double* __restrict__ ll, const int64_t* __restrict__ labels,
     const int64_t* __restrict__ act_lens, const int64_t* __restrict__ label_lens, const float* __restrict__ grad_scale,
     int grad_scale_stride, float grad_mul, float* __restrict__ coef, int T, int U, int V, int blank, int ND, int Us,
     int A, int CS, float lambda, float clamp, long long cells) {
-  const long long c = (long long)blockIdx.x * blockDim.x + threadIdx.x;
-  if (c >= cells) return;
-  const int u = (int)(c % U);
-  const long long bt = c / U;
-  const int t = (int)(bt % T);
-  const int b = (int)(bt / T);
+  // one workgroup per skewed row (b, n = t + u), one thread per column: the lattice reads of a wave
+  // are then consecutive addresses (a thread per cell in [B,T,U] order strides by a whole row + 1)
+  const int u = threadIdx.x, b = (int)(blockIdx.x / (unsigned)ND), n = (int)(blockIdx.x - (unsigned)b * (unsigned)ND);
+  const int t = n - u;
+  if (u >= U || t < 0 || t >= T) return;
+  const long long c = ((long long)b * T + t) * U + u;
+  (void)cells;
   const int Tb = clampi(act_lens[b], 1, T);
   const int Ub = clampi(label_lens[b] + 1, 1, U);
   float* out = coef + (size_t)c * CS;
@@ -1208,18 +1206,19 @@ __global__ __launch_bounds__(256) void rnnt_cell_kernel(
                             lambda, clamp));
 }
 
-__global__ __launch_bounds__(256) void tdt_cell_kernel(
+__global__ __launch_bounds__(1024) void tdt_cell_kernel(
     const float* __restrict__ denom, const float* __restrict__ arcs, const double* __restrict__ alphas,
     const double* __restrict__ betas, const double* __restrict__ ll, const int64_t* __restrict__ labels,
     const int64_t* __restrict__ act_lens, const int64_t* __restrict__ label_lens, const float* __restrict__ grad_scale,
     int grad_scale_stride, float grad_mul, float* __restrict__ coef, int T, int U, int V, int blank, int ND, int Us,
     int A, int CS, float lambda, float clamp, long long cells, TdtParams prm) {
-  const long long c = (long long)blockIdx.x * blockDim.x + threadIdx.x;
-  if (c >= cells) return;
-  const int u = (int)(c % U);
-  const long long bt = c / U;
-  const int t = (int)(bt % T);
-  const int b = (int)(bt / T);
+  // one workgroup per skewed row (b, n = t + u), one thread per column: the lattice reads of a wave
+  // are then consecutive addresses (a thread per cell in [B,T,U] order strides by a whole row + 1)
+  const int u = threadIdx.x, b = (int)(blockIdx.x / (unsigned)ND), n = (int)(blockIdx.x - (unsigned)b * (unsigned)ND);
+  const int t = n - u;
+  if (u >= U || t < 0 || t >= T) return;
+  const long long c = ((long long)b * T + t) * U + u;
+  (void)cells;
   const int Tb = clampi(act_lens[b], 1, T);
   const int Ub = clampi(label_lens[b] + 1, 1, U);
   float* out = coef + (size_t)c * CS;
@@ -1471,18 +1470,19 @@ __global__ __launch_bounds__(MAXT) void multiblank_lattice_kernel(
 // Per-cell coefficients of the multi-blank gradient (gpu_rnnt_kernel.py:727-885): the record of the
 // RNNT/TDT cell kernels, plus in out[kCoefBase + i] the FINISHED gradient entry of big blank i
 // (clamped and scaled), which multiblank_fixup_kernel stores over what the gradient pass put there.
-__global__ __launch_bounds__(256) void multiblank_cell_kernel(
+__global__ __launch_bounds__(1024) void multiblank_cell_kernel(
     const float* __restrict__ denom, const float* __restrict__ arcs,
     const double* __restrict__ alphas, const double* __restrict__ betas, const double* __restrict__ ll,
     const int64_t* __restrict__ labels, const int64_t* __restrict__ act_lens, const int64_t* __restrict__ label_lens,
     const float* __restrict__ grad_scale, int grad_scale_stride, float grad_mul, float* __restrict__ coef, int T, int U,
     int V, int blank, int ND, int Us, int A, int CS, float lambda, float clamp, long long cells, MbParams prm) {
-  const long long c = (long long)blockIdx.x * blockDim.x + threadIdx.x;
-  if (c >= cells) return;
-  const int u = (int)(c % U);
-  const long long bt = c / U;
-  const int t = (int)(bt % T);
-  const int b = (int)(bt / T);
+  // one workgroup per skewed row (b, n = t + u), one thread per column: the lattice reads of a wave
+  // are then consecutive addresses (a thread per cell in [B,T,U] order strides by a whole row + 1)
+  const int u = threadIdx.x, b = (int)(blockIdx.x / (unsigned)ND), n = (int)(blockIdx.x - (unsigned)b * (unsigned)ND);
+  const int t = n - u;
+  if (u >= U || t < 0 || t >= T) return;
+  const long long c = ((long long)b * T + t) * U + u;
+  (void)cells;
   const int Tb = clampi(act_lens[b], 1, T);
   const int Ub = clampi(label_lens[b] + 1, 1, U);
   float* out = coef + (size_t)c * CS;
@@ -2684,9 +2684,8 @@ int run_grad_stream(const Common& c, void* grads, int flags, bool fused, const S
 int run_rnnt_cells(const Common& c, const ScaleArg& sc, float lambda, float clamp) {
   const Layout& L = c.L;
   const long long cells = (long long)c.B * c.T * c.U;
-  const unsigned grid = (unsigned)((cells + 255) / 256);
   ProfScope prof(MI_PROFILE_CELL, c.stream);
-  hipLaunchKernelGGL(rnnt_cell_kernel, dim3(grid), dim3(256), 0, c.stream, (const float*)(c.ws + L.off_denom),
+  hipLaunchKernelGGL(rnnt_cell_kernel, dim3((unsigned)(L.ND * c.B)), dim3(L.Us), 0, c.stream, (const float*)(c.ws + L.off_denom),
                      (const float*)(c.ws + L.off_arcs), (const double*)(c.ws + L.off_alphas),
                      (const double*)(c.ws + L.off_betas), (const double*)(c.ws + L.off_ll), c.labels, c.act_lens,
                      c.label_lens, sc.ptr, sc.stride, sc.mul, (float*)(c.ws + L.off_coef), c.T, c.U, c.V, c.blank, L.ND,
@@ -2697,9 +2696,8 @@ int run_rnnt_cells(const Common& c, const ScaleArg& sc, float lambda, float clam
 int run_tdt_cells(const Common& c, const ScaleArg& sc, float lambda, float clamp, const TdtParams& prm) {
   const Layout& L = c.L;
   const long long cells = (long long)c.B * c.T * c.U;
-  const unsigned grid = (unsigned)((cells + 255) / 256);
   ProfScope prof(MI_PROFILE_CELL, c.stream);
-  hipLaunchKernelGGL(tdt_cell_kernel, dim3(grid), dim3(256), 0, c.stream, (const float*)(c.ws + L.off_denom),
+  hipLaunchKernelGGL(tdt_cell_kernel, dim3((unsigned)(L.ND * c.B)), dim3(L.Us), 0, c.stream, (const float*)(c.ws + L.off_denom),
                      (const float*)(c.ws + L.off_arcs), (const double*)(c.ws + L.off_alphas),
                      (const double*)(c.ws + L.off_betas), (const double*)(c.ws + L.off_ll), c.labels, c.act_lens,
                      c.label_lens, sc.ptr, sc.stride, sc.mul, (float*)(c.ws + L.off_coef), c.T, c.U, c.V, c.blank, L.ND,
@@ -2765,9 +2763,8 @@ int run_multiblank_lattice(const Common& c, float* costs, float lambda, int with
 int run_multiblank_cells(const Common& c, const ScaleArg& sc, float lambda, float clamp, const MbParams& prm) {
   const Layout& L = c.L;
   const long long cells = (long long)c.B * c.T * c.U;
-  const unsigned grid = (unsigned)((cells + 255) / 256);
   ProfScope prof(MI_PROFILE_CELL, c.stream);
-  hipLaunchKernelGGL(multiblank_cell_kernel, dim3(grid), dim3(256), 0, c.stream, (const float*)(c.ws + L.off_denom),
+  hipLaunchKernelGGL(multiblank_cell_kernel, dim3((unsigned)(L.ND * c.B)), dim3(L.Us), 0, c.stream, (const float*)(c.ws + L.off_denom),
                      (const float*)(c.ws + L.off_arcs), (const double*)(c.ws + L.off_alphas),
                      (const double*)(c.ws + L.off_betas), (const double*)(c.ws + L.off_ll), c.labels, c.act_lens,
                      c.label_lens, sc.ptr, sc.stride, sc.mul, (float*)(c.ws + L.off_coef), c.T, c.U, c.V, c.blank, L.ND,
