@@ -13,7 +13,10 @@ lengths), inputs already in HBM.  Prints ONE JSON line:
   kernels      mean duration of each pipeline kernel over the timed steps (ms)
   copy_probe   bandwidth a plain device copy reaches on this GPU (GB/s, read + write)
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload 0..5] [--no-cpu-baseline]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload 0..5] [--op loss|logprobs] [--no-cpu-baseline]
+
+--op logprobs measures the compact log-prob op on the same tensors instead (speech_amd.k2.rnnt_logprobs
+forward + backward with given upstream gradients; RNNT workloads only).
 """
 
 import argparse
@@ -44,6 +47,7 @@ def parse_args():
     ap.add_argument("--steps", type=int, default=30)
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--workload", type=int, default=1, help="index into speech_amd.synthetic.CONFIGS (1 = north star)")
+    ap.add_argument("--op", choices=["loss", "logprobs"], default="loss")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--cpu-sample-utterances", type=int, default=16)
     return ap.parse_args()
@@ -82,6 +86,30 @@ def cpu_baseline(cfg, acts, labels, act_lens, label_lens, n_utt):
     }
 
 
+def cpu_baseline_logprobs(cfg, acts, labels, act_lens, label_lens, g_target, g_blank, n_utt):
+    """The numpy restatement of the compact log-prob op (forward + backward), one host thread."""
+    import oracle
+
+    n_utt = min(n_utt, cfg.B)
+    x = acts[:n_utt].float().cpu().numpy()
+    lab = labels[:n_utt].cpu().numpy()
+    al = act_lens[:n_utt].cpu().numpy()
+    ll = label_lens[:n_utt].cpu().numpy()
+    gt, gb = g_target[:n_utt].cpu().numpy(), g_blank[:n_utt].cpu().numpy()
+    t0 = time.perf_counter()
+    oracle.rnnt_logprobs(x, lab, cfg.blank, al, ll)
+    oracle.rnnt_logprobs_grad(x, lab, cfg.blank, gt, gb, al, ll)
+    dt = time.perf_counter() - t0
+    return {
+        "value": x.size / dt,
+        "unit": "logit elems/s",
+        "cores": 1,
+        "kind": "port",
+        "sample": f"first {n_utt} of {cfg.B} utterances of the same batch, full T x U x V, forward + backward, "
+                  f"{dt:.2f} s wall (numpy, float64)",
+    }  # fmt: skip
+
+
 def main():
     args = parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
@@ -117,6 +145,27 @@ def main():
         costs = loss(acts, labels, act_lens, label_lens)
         costs.sum().backward()
         return costs
+
+    logprobs = args.op == "logprobs"
+    if logprobs:
+        if cfg.D or cfg.big_blank_durations:
+            print("bench.py: --op logprobs runs on the RNNT workloads (0, 1, 2, 4)", file=sys.stderr)
+            sys.exit(2)
+        from speech_amd.k2 import rnnt_logprobs
+
+        g_target = torch.rand(cfg.B, cfg.T, cfg.U, device=dev)
+        g_blank = torch.rand(cfg.B, cfg.T, cfg.U, device=dev)
+        # forward reads the valid rows and writes two score arrays; backward reads them, the two upstream
+        # gradients and the valid rows again and writes every gradient element
+        s_in = acts.element_size()
+        nbytes = dict(nbytes)
+        nbytes["total"] = 2 * nbytes["c_valid"] * cfg.V * s_in + nbytes["cells"] * cfg.V * s_in + 16 * nbytes["cells"]
+
+        def step():  # noqa: F811
+            acts.grad = None
+            target_scores, blank_scores = rnnt_logprobs(acts, labels, cfg.blank, act_lens, label_lens)
+            torch.autograd.backward([target_scores, blank_scores], [g_target, g_blank])
+            return blank_scores
 
     for _ in range(args.warmup):
         step()
@@ -172,11 +221,15 @@ def main():
     grad_avg_s = grad_ms * 1e-3 / max(grad_n, 1)
     # with the padding zero-filled by its own kernel during forward, the gradient pass reads and
     # writes the valid rows only
-    overlap = rnnt_pytorch.OVERLAP_PADDING
+    overlap = rnnt_pytorch.OVERLAP_PADDING and not logprobs
+    if logprobs:  # the op's backward always streams the coefficient records of its own cell kernel
+        plan["lattice"], plan["cells"] = "none", "logprobs_export_kernel + logprobs_cell_kernel"
+        plan["gradient"] = plan["gradient"].replace("fused>", "coef>")
     grad_bytes = nbytes["grad_valid"] if overlap else nbytes["grad_stream"]
     achieved = grad_bytes / grad_avg_s / 1e9
     result = {
-        "metric": "RNNT/TDT loss fwd+bwd: logit elems/s and achieved HBM GB/s vs peak",
+        "metric": ("compact log-prob op fwd+bwd: logit elems/s and achieved HBM GB/s vs peak" if logprobs else
+                   "RNNT/TDT loss fwd+bwd: logit elems/s and achieved HBM GB/s vs peak"),
         "value": cfg.elems / (ms_per_step * 1e-3),
         "unit": "logit elems/s",
         "n_gpus": 1,
@@ -189,7 +242,7 @@ def main():
         "dtype": {torch.float32: "f32", torch.bfloat16: "bf16", torch.float16: "f16"}[cfg.dtype],
         "data": "synthetic",
         "config": {
-            "workload": cfg.name,
+            "workload": cfg.name + ("_logprobs" if logprobs else ""),
             "B": cfg.B, "T": cfg.T, "U": cfg.U, "V": cfg.V, "D": cfg.D,
             "valid_cells": nbytes["c_valid"], "cells": nbytes["cells"],
             "fastemit_lambda": cfg.fastemit_lambda, "clamp": cfg.clamp, "sigma": cfg.sigma,
@@ -207,7 +260,7 @@ def main():
             "peak": HBM_PEAK_GBPS,
             "unit": "GB/s",
             "frac": achieved / HBM_PEAK_GBPS,
-            "traffic": MEASURED_TRAFFIC_BYTES.get((cfg.name, overlap)),
+            "traffic": None if logprobs else MEASURED_TRAFFIC_BYTES.get((cfg.name, overlap)),
             "algorithmic_bytes_per_launch": grad_bytes,
             "padding_zero_filled_by": "zero_padding_kernel (second stream, during forward)" if overlap else "this kernel",
             "avg_launch_ms": grad_avg_s * 1e3,
@@ -217,7 +270,11 @@ def main():
         "plan": plan,
         "copy_probe_GBps": copy_gbps,
     }  # fmt: skip
-    if not args.no_cpu_baseline:
+    if not args.no_cpu_baseline and logprobs:
+        result["cpu_baseline"] = cpu_baseline_logprobs(
+            cfg, acts.detach(), labels, act_lens, label_lens, g_target, g_blank, min(args.cpu_sample_utterances, 8)
+        )
+    elif not args.no_cpu_baseline:
         result["cpu_baseline"] = cpu_baseline(
             cfg, acts.detach(), labels, act_lens, label_lens, args.cpu_sample_utterances
         )

@@ -172,6 +172,30 @@ int mi_tdt_lattice(const int64_t* act_lens, const int64_t* label_lens, float* co
 int mi_transducer_zero_padding(void* grads, int act_dtype, const int64_t* act_lens, const int64_t* label_lens, int B,
                                int T, int U, int VD, void* stream);
 
+/* ---- compact log-prob op ---------------------------------------------------------------
+ * Replaces rnnt_logprobs_triton (nemo/collections/asr/parts/k2/rnnt_logprobs_triton.py:20-228), the
+ * producer of the graph-transducer losses' inputs (parts/k2/graph_transducer.py:517).
+ *
+ * forward:  target_scores[b,t,u] = log_softmax(logits[b,t,u,:])[targets[b,u]]   (u <  target_lens[b])
+ *           blank_scores [b,t,u] = log_softmax(logits[b,t,u,:])[blank]          (u <= target_lens[b])
+ *           for t < source_lens[b]; every other entry of the two float32 [B,T,U] arrays is set to 0
+ *           (the reference leaves them at the zeros it allocated, :148-149).  U = max target length + 1.
+ *           The workspace (mi_transducer_workspace_bytes(B, T, U, 0)) keeps the denominators.
+ * backward: grad_logits[b,t,u,v] = -softmax_v * (gb + gt) + [v = blank] gb + [v = target] gt with
+ *           gb = grad_blank_scores[b,t,u], gt = grad_target_scores[b,t,u] (0 where there is no target);
+ *           when target == blank only gt is added, as the reference does (:118-122).  Cells outside
+ *           an utterance get 0.  have_forward_state != 0: `workspace` is the one the forward call
+ *           filled for the same inputs; 0: the denominators are recomputed first (what the
+ *           reference always does, :90-104), at the price of one more read of the logits.
+ * Lengths and targets are int64 device arrays ([B], [B,U-1]); logits/grad_logits share act_dtype. */
+int mi_rnnt_logprobs_forward(const void* logits, int act_dtype, const int64_t* targets, const int64_t* source_lens,
+                             const int64_t* target_lens, float* target_scores, float* blank_scores, int B, int T, int U,
+                             int V, int blank, void* workspace, size_t workspace_bytes, void* stream);
+int mi_rnnt_logprobs_backward(const void* logits, int act_dtype, const int64_t* targets, const int64_t* source_lens,
+                              const int64_t* target_lens, const float* grad_target_scores,
+                              const float* grad_blank_scores, void* grad_logits, int have_forward_state, int B, int T,
+                              int U, int V, int blank, void* workspace, size_t workspace_bytes, void* stream);
+
 /* Stage-level read-out for kernel parity tests (the reference tests launch each
  * kernel on its own, tests/collections/asr/numba/rnnt_loss/utils/test_gpu_rnnt_kernel.py):
  * copies what the last forward call left in `workspace` into plain [B,T,U] float32

@@ -176,3 +176,19 @@ def multiblank_loss(
     if status != 0:
         raise RuntimeError("oracle_multiblank_loss: invalid value")
     return costs, grads, dict(denom=denom, alphas=alphas, betas=betas, ll_forward=llf, ll_backward=llb)
+
+
+def rnnt_logprobs(logits, targets, blank, source_lens=None, target_lens=None):
+    """Compact log-prob op, forward (numpy restatement; see transducer_numpy.rnnt_logprobs)."""
+    from oracle import transducer_numpy
+
+    return transducer_numpy.rnnt_logprobs(logits, targets, blank, source_lens, target_lens)
+
+
+def rnnt_logprobs_grad(logits, targets, blank, grad_target_scores, grad_blank_scores, source_lens=None, target_lens=None):
+    """Compact log-prob op, backward (numpy restatement; see transducer_numpy.rnnt_logprobs_grad)."""
+    from oracle import transducer_numpy
+
+    return transducer_numpy.rnnt_logprobs_grad(
+        logits, targets, blank, grad_target_scores, grad_blank_scores, source_lens, target_lens
+    )

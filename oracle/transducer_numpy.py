@@ -25,6 +25,9 @@ How each function is pinned (tests/test_oracle_*.py):
                     path, torch autograd of an alpha-only recursion,
                     llForward == beta(0,0) ........................... pinned
   multiblank_* FastEmit  derived only, as for TDT
+  rnnt_logprobs*    torch log_softmax + gather (the reference's own etalon,
+                    parts/k2/rnnt_logprobs.py:19-48) and torch autograd
+                    through it, in float64 ........................... pinned
 
 The loops are slow on purpose (clarity first): use them at lattice sizes up to
 a few thousand cells; oracle/transducer_cpu.c is the fast restatement.
@@ -563,3 +566,63 @@ def multiblank_loss(
         llf[b], llb[b] = ll, ll_b
         costs[b] = -ll * dtype(1.0 + fastemit_lambda)
     return costs, grads, dict(denom=denom, alphas=alphas, betas=betas, ll_forward=llf, ll_backward=llb)
+
+
+# ----------------------------------------------------------------------------------------
+# Compact log-prob op (nemo/collections/asr/parts/k2/rnnt_logprobs_triton.py)
+# ----------------------------------------------------------------------------------------
+def _logprobs_masks(B, T, U, source_lens, target_lens):
+    source_lens = np.full(B, T) if source_lens is None else np.asarray(source_lens)
+    target_lens = np.full(B, U - 1) if target_lens is None else np.asarray(target_lens)
+    t = np.arange(T)[None, :, None]
+    u = np.arange(U)[None, None, :]
+    in_time = t < source_lens[:, None, None]
+    cell = in_time & (u <= target_lens[:, None, None])  # :46-48: rows with t >= len or u > target_len are skipped
+    has_target = in_time & (u < target_lens[:, None, None])  # :64
+    return cell, has_target
+
+
+def rnnt_logprobs(logits, targets, blank, source_lens=None, target_lens=None):
+    """(target_scores, blank_scores), [B,T,U] each; rnnt_logprobs_triton.py:20-69.
+
+    log-softmax over the last axis, read at the target id of column u and at the blank id; entries of
+    skipped rows, and target entries of columns without a target, stay 0 (:148-149).
+    """
+    x = np.asarray(logits, dtype=np.float64)
+    B, T, U, V = x.shape
+    targets = np.asarray(targets).reshape(B, U - 1)
+    cell, has_target = _logprobs_masks(B, T, U, source_lens, target_lens)
+    m = x.max(axis=-1)
+    log_norm = m + np.log(np.exp(x - m[..., None]).sum(axis=-1))
+    ids = np.concatenate([targets, np.zeros((B, 1), dtype=targets.dtype)], axis=1)  # column U-1: any id, masked below
+    picked = np.take_along_axis(x, np.broadcast_to(ids[:, None, :, None], (B, T, U, 1)), axis=-1)[..., 0]
+    target_scores = np.where(has_target, picked - log_norm, 0.0)
+    blank_scores = np.where(cell, x[..., blank] - log_norm, 0.0)
+    return target_scores, blank_scores
+
+
+def rnnt_logprobs_grad(logits, targets, blank, grad_target_scores, grad_blank_scores, source_lens=None, target_lens=None):
+    """Gradient of the logits given those of the two score arrays; rnnt_logprobs_triton.py:72-127.
+
+    g_v = -softmax_v * (gb + gt), plus gb at the blank id, plus gt at the target id -- and where the
+    target id IS the blank id the second `where` (:122) replaces the first, so only gt is added there.
+    Skipped rows stay 0 (:211).
+    """
+    x = np.asarray(logits, dtype=np.float64)
+    B, T, U, V = x.shape
+    targets = np.asarray(targets).reshape(B, U - 1)
+    cell, has_target = _logprobs_masks(B, T, U, source_lens, target_lens)
+    gb = np.where(cell, np.asarray(grad_blank_scores, dtype=np.float64), 0.0)
+    gt = np.where(has_target, np.asarray(grad_target_scores, dtype=np.float64), 0.0)
+    m = x.max(axis=-1, keepdims=True)
+    e = np.exp(x - m)
+    softmax = e / e.sum(axis=-1, keepdims=True)
+    grad = -softmax * (gb + gt)[..., None]
+    base = grad.copy()
+    grad[..., blank] = base[..., blank] + gb
+    ids = np.concatenate([targets, np.zeros((B, 1), dtype=targets.dtype)], axis=1)
+    idx = np.broadcast_to(ids[:, None, :, None], (B, T, U, 1))
+    at_target = np.take_along_axis(base, idx, axis=-1)[..., 0] + gt
+    current = np.take_along_axis(grad, idx, axis=-1)[..., 0]
+    np.put_along_axis(grad, idx, np.where(has_target, at_target, current)[..., None], axis=-1)
+    return np.where(cell[..., None], grad, 0.0)

@@ -1206,6 +1206,67 @@ __global__ __launch_bounds__(1024) void rnnt_cell_kernel(
                             lambda, clamp));
 }
 
+// ----------------------------------------------------------------------------------------
+// Compact log-prob op (parts/k2/rnnt_logprobs_triton.py:20-228): target and blank log-probs of every
+// lattice cell as plain [B,T,U] float32 arrays, and the gradient of the logits given the gradients of
+// those two arrays.  The forward is the denominator pass plus this read-out of its arc planes; the
+// backward turns the two upstream gradients into the per-cell coefficient records of the streaming
+// gradient pass:  g_v = -p_v * (gb + gt) + [v = blank] gb + [v = target] gt  (:118-122; with
+// target == blank the target term alone is added, as there).  One workgroup per skewed row, one
+// thread per column.
+// ----------------------------------------------------------------------------------------
+__global__ __launch_bounds__(1024) void logprobs_export_kernel(const float* __restrict__ arcs,
+                                                              const int64_t* __restrict__ act_lens,
+                                                              const int64_t* __restrict__ label_lens,
+                                                              float* __restrict__ target_scores,
+                                                              float* __restrict__ blank_scores, int T, int U, int ND,
+                                                              int Us, int A) {
+  const int u = threadIdx.x, b = (int)(blockIdx.x / (unsigned)ND), n = (int)(blockIdx.x - (unsigned)b * (unsigned)ND);
+  const int t = n - u;
+  if (u >= U || t < 0 || t >= T) return;
+  const size_t c = ((size_t)b * T + t) * U + u;
+  const int Tb = clampi(act_lens[b], 1, T);
+  const int Ub = clampi(label_lens[b] + 1, 1, U);
+  const bool valid = t < Tb && u < Ub;
+  const size_t base = (size_t)(b * ND + n) * A * Us + u;
+  const float lpb = arcs[base], lpl = arcs[base + Us];
+  blank_scores[c] = valid ? lpb : 0.f;                  // cells outside the utterance stay 0 (:148-149)
+  target_scores[c] = (valid && u < Ub - 1) ? lpl : 0.f;  // and so does the column without a target
+}
+
+__global__ __launch_bounds__(1024) void logprobs_cell_kernel(
+    const float* __restrict__ denom, const float* __restrict__ arcs, const int64_t* __restrict__ labels,
+    const int64_t* __restrict__ act_lens, const int64_t* __restrict__ label_lens,
+    const float* __restrict__ grad_target_scores, const float* __restrict__ grad_blank_scores,
+    float* __restrict__ coef, int T, int U, int V, int blank, int ND, int Us, int A, int CS) {
+  const int u = threadIdx.x, b = (int)(blockIdx.x / (unsigned)ND), n = (int)(blockIdx.x - (unsigned)b * (unsigned)ND);
+  const int t = n - u;
+  if (u >= U || t < 0 || t >= T) return;
+  const size_t c = ((size_t)b * T + t) * U + u;
+  const int Tb = clampi(act_lens[b], 1, T);
+  const int Ub = clampi(label_lens[b] + 1, 1, U);
+  float* out = coef + c * CS;
+  if (t >= Tb || u >= Ub) {
+    out[5] = __int_as_float(-2);
+    return;
+  }
+  const size_t base = (size_t)(b * ND + n) * A * Us + u;
+  const bool has_target = u < Ub - 1;
+  const int lab = has_target ? clampi(labels[(size_t)b * (U - 1) + u], 0, V - 1) : -1;
+  const float gb = grad_blank_scores[c];
+  const float gt = has_target ? grad_target_scores[c] : 0.f;
+  const float sum = gb + gt;
+  RowCoef rc;
+  rc.dl2 = denom[c] * kLog2e;
+  rc.W = -sum;
+  rc.cb = INFINITY;
+  rc.gB = gb - __expf(arcs[base]) * sum;
+  rc.gL = has_target ? gt - __expf(arcs[base + Us]) * sum : 0.f;
+  if (lab == blank) rc.gB = rc.gL;
+  rc.lab = lab;
+  write_coef(out, rc);
+}
+
 __global__ __launch_bounds__(1024) void tdt_cell_kernel(
     const float* __restrict__ denom, const float* __restrict__ arcs, const double* __restrict__ alphas,
     const double* __restrict__ betas, const double* __restrict__ ll, const int64_t* __restrict__ labels,
@@ -2693,6 +2754,25 @@ int run_rnnt_cells(const Common& c, const ScaleArg& sc, float lambda, float clam
   return launch_status();
 }
 
+int run_logprobs_export(const Common& c, float* target_scores, float* blank_scores) {
+  const Layout& L = c.L;
+  ProfScope prof(MI_PROFILE_CELL, c.stream);
+  hipLaunchKernelGGL(logprobs_export_kernel, dim3((unsigned)(L.ND * c.B)), dim3(L.Us), 0, c.stream,
+                     (const float*)(c.ws + L.off_arcs), c.act_lens, c.label_lens, target_scores, blank_scores, c.T,
+                     c.U, L.ND, L.Us, L.A);
+  return launch_status();
+}
+
+int run_logprobs_cells(const Common& c, const float* grad_target_scores, const float* grad_blank_scores) {
+  const Layout& L = c.L;
+  ProfScope prof(MI_PROFILE_CELL, c.stream);
+  hipLaunchKernelGGL(logprobs_cell_kernel, dim3((unsigned)(L.ND * c.B)), dim3(L.Us), 0, c.stream,
+                     (const float*)(c.ws + L.off_denom), (const float*)(c.ws + L.off_arcs), c.labels, c.act_lens,
+                     c.label_lens, grad_target_scores, grad_blank_scores, (float*)(c.ws + L.off_coef), c.T, c.U, c.V,
+                     c.blank, L.ND, L.Us, L.A, L.CS);
+  return launch_status();
+}
+
 int run_tdt_cells(const Common& c, const ScaleArg& sc, float lambda, float clamp, const TdtParams& prm) {
   const Layout& L = c.L;
   const long long cells = (long long)c.B * c.T * c.U;
@@ -2791,7 +2871,7 @@ int run_multiblank_fixup(const Common& c, void* grads, const MbParams& prm) {
 // ----------------------------------------------------------------------------------------
 extern "C" {
 
-int mi_transducer_abi_version(void) { return 7; }
+int mi_transducer_abi_version(void) { return 8; }
 
 int mi_transducer_workspace_bytes(int B, int T, int U, int D, size_t* out_bytes) {
   Layout L;
@@ -2940,6 +3020,33 @@ int mi_multiblank_loss(const void* acts, int act_dtype, const int64_t* labels, c
   return mi_multiblank_backward(acts, act_dtype, labels, act_lens, label_lens, grads, grad_scale, grad_scale_stride,
                                 grad_mul, B, T, U, V, num_big_blanks, big_blank_durations_host, blank, fastemit_lambda,
                                 clamp, sigma, workspace, workspace_bytes, stream);
+}
+
+int mi_rnnt_logprobs_forward(const void* logits, int act_dtype, const int64_t* targets, const int64_t* source_lens,
+                             const int64_t* target_lens, float* target_scores, float* blank_scores, int B, int T, int U,
+                             int V, int blank, void* workspace, size_t workspace_bytes, void* stream) {
+  Common c;
+  if (!target_scores || !blank_scores) return MI_TRANSDUCER_INVALID_VALUE;
+  int st = check_common(logits, act_dtype, targets, source_lens, target_lens, B, T, U, V, 0, blank, workspace,
+                        workspace_bytes, stream, &c);
+  if (st) return st;
+  if ((st = run_denom(c))) return st;
+  return run_logprobs_export(c, target_scores, blank_scores);
+}
+
+int mi_rnnt_logprobs_backward(const void* logits, int act_dtype, const int64_t* targets, const int64_t* source_lens,
+                              const int64_t* target_lens, const float* grad_target_scores,
+                              const float* grad_blank_scores, void* grad_logits, int have_forward_state, int B, int T,
+                              int U, int V, int blank, void* workspace, size_t workspace_bytes, void* stream) {
+  Common c;
+  if (!grad_target_scores || !grad_blank_scores || !grad_logits) return MI_TRANSDUCER_INVALID_VALUE;
+  int st = check_common(logits, act_dtype, targets, source_lens, target_lens, B, T, U, V, 0, blank, workspace,
+                        workspace_bytes, stream, &c);
+  if (st) return st;
+  if (!have_forward_state && (st = run_denom(c))) return st;
+  if ((st = run_logprobs_cells(c, grad_target_scores, grad_blank_scores))) return st;
+  const ScaleArg sc = {nullptr, 0, 1.f};
+  return run_grad_stream(c, grad_logits, 0, false, sc, 0.f, 0.f);
 }
 
 int mi_transducer_export_lattice(const void* workspace, size_t workspace_bytes, const int64_t* act_lens,
