@@ -196,6 +196,22 @@ int mi_rnnt_logprobs_backward(const void* logits, int act_dtype, const int64_t* 
                               const float* grad_blank_scores, void* grad_logits, int have_forward_state, int B, int T,
                               int U, int V, int blank, void* workspace, size_t workspace_bytes, void* stream);
 
+/* ---- joint projection fused into the forward pass --------------------------------------
+ * Replaces RNNTJoint.joint_after_projection followed by the loss forward
+ * (nemo/collections/asr/modules/rnnt.py:1707-1724 and :1573-1578) for the default joint network
+ * (ReLU, no dropout, Linear(H -> V); :1759-1777): the [B,T,U,V] tensor is never written.
+ *   f [B,T,H], g [B,U,H]: bf16, the projected encoder / prediction-network outputs (16-byte aligned);
+ *   weight [V,H], bias [V] (nullable): float32 or bf16 (weight_dtype), the final Linear layer;
+ *   logits = relu(f[b,t] + g[b,u]) . weight^T + bias with bf16 operands and float32 accumulation
+ *   (what the reference computes under bf16 autocast, minus its rounding of the logits to bf16).
+ * costs[b] as mi_rnnt_forward; the workspace (mi_joint_workspace_bytes) ends up holding the same
+ * lattice state.  H must be 512 or 640; V any. */
+int mi_joint_workspace_bytes(int B, int T, int U, int H, int V, size_t* out_bytes);
+int mi_joint_rnnt_forward(const void* f, const void* g, const void* weight, const void* bias, int weight_dtype,
+                          const int64_t* labels, const int64_t* act_lens, const int64_t* label_lens, float* costs,
+                          int B, int T, int U, int H, int V, int blank, float fastemit_lambda, int with_betas,
+                          void* workspace, size_t workspace_bytes, void* stream);
+
 /* Stage-level read-out for kernel parity tests (the reference tests launch each
  * kernel on its own, tests/collections/asr/numba/rnnt_loss/utils/test_gpu_rnnt_kernel.py):
  * copies what the last forward call left in `workspace` into plain [B,T,U] float32
