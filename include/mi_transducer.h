@@ -209,8 +209,24 @@ int mi_rnnt_logprobs_backward(const void* logits, int act_dtype, const int64_t* 
 int mi_joint_workspace_bytes(int B, int T, int U, int H, int V, size_t* out_bytes);
 int mi_joint_rnnt_forward(const void* f, const void* g, const void* weight, const void* bias, int weight_dtype,
                           const int64_t* labels, const int64_t* act_lens, const int64_t* label_lens, float* costs,
-                          int B, int T, int U, int H, int V, int blank, float fastemit_lambda, int with_betas,
-                          void* workspace, size_t workspace_bytes, void* stream);
+                          int* tile_count, int B, int T, int U, int H, int V, int blank, float fastemit_lambda,
+                          int with_betas, void* workspace, size_t workspace_bytes, void* stream);
+
+/* Backward of the fused joint, first half: the logits are recomputed tile by tile exactly as in the forward call
+ * and turned into their gradient (gpu_rnnt_kernel.py:340-403 with grad_scale folded in, as mi_rnnt_backward), which
+ * is stored as bf16 for the two matrix products that finish the job (d weight = dlogits^T . h, d hidden =
+ * dlogits . weight): one row per lattice cell in the kernel's tile order -- utterance by utterance, cell t*U_b + u,
+ * each utterance padded to a multiple of 128 rows with zero rows -- and padded_vocabulary(V) columns, the ones
+ * beyond V zero.  row_ft / row_gu receive, per row, the flat indices b*T + t and b*U + u of the cell's rows in f
+ * and g (0 for the zero rows).  `tiles` is the number of 128-row tiles the three buffers hold: at least what
+ * mi_joint_rnnt_forward wrote to tile_count (device int32, nullable there), whose workspace this call needs
+ * unchanged (forward with with_betas != 0). */
+int mi_joint_padded_vocabulary(int V);
+int mi_joint_rnnt_backward_logits(const void* f, const void* g, const int64_t* labels, const int64_t* act_lens,
+                                  const int64_t* label_lens, void* dlogits, int64_t* row_ft, int64_t* row_gu,
+                                  int tiles, const float* grad_scale, int grad_scale_stride, float grad_mul, int B,
+                                  int T, int U, int H, int V, int blank, float fastemit_lambda, float clamp,
+                                  void* workspace, size_t workspace_bytes, void* stream);
 
 /* Stage-level read-out for kernel parity tests (the reference tests launch each
  * kernel on its own, tests/collections/asr/numba/rnnt_loss/utils/test_gpu_rnnt_kernel.py):

@@ -1,10 +1,18 @@
-"""Joint network + RNNT loss forward in one pass over the lattice cells.
+"""Joint network + RNNT loss without the [B,T,U,V] tensor.
 
 The reference computes `joint_net(f.unsqueeze(2) + g.unsqueeze(1))` -- ReLU, Linear(H -> V) -- into a
-[B,T,U,V] tensor (nemo/collections/asr/modules/rnnt.py:1707-1724, :1759-1777) and hands it to the
-loss (:1573-1578).  `joint_rnnt_forward` takes the joint network's inputs instead and returns the same
-per-utterance costs; the logits exist only tile by tile inside the kernel (bf16 operands, float32
-accumulation, as under bf16 autocast).
+[B,T,U,V] tensor (nemo/collections/asr/modules/rnnt.py:1707-1724, joint_net built at :1759-1777) and hands it
+to the loss (:1573-1578); autograd then keeps that tensor and a gradient of the same size.  Here
+
+  forward   one kernel forms the logits tile by tile on the matrix cores (bf16 operands, float32 accumulation: the
+            arithmetic of bf16 autocast) and keeps only each cell's log-softmax denominator and its blank / label
+            log-probs; the lattice kernel turns those into the costs;
+  backward  the same kernel recomputes the logits and writes their gradient as bf16, one row per VALID lattice
+            cell (padded cells are never touched); two library GEMMs give d weight and d hidden, and d hidden is
+            summed over u into d f and over t into d g.
+
+`joint_rnnt_loss` is differentiable in f, g, weight and bias; `joint_rnnt_forward` is the no-grad form.
+Limits: ReLU joint without dropout (the reference's default `jointnet.activation`), H in {512, 640}.
 """
 
 import ctypes
@@ -14,7 +22,7 @@ import torch
 from speech_amd import _native
 from speech_amd.rnnt_loss.rnnt import _labels_ptr, _ptr, _require_gpu, _stream
 
-__all__ = ["joint_rnnt_forward"]
+__all__ = ["joint_rnnt_forward", "joint_rnnt_loss", "JointRNNTLoss"]
 
 
 def joint_workspace(B, T, U, H, V, device):
@@ -27,36 +35,115 @@ def joint_workspace(B, T, U, H, V, device):
     return torch.empty(nbytes.value, dtype=torch.uint8, device=device)
 
 
-def joint_rnnt_forward(f, g, weight, bias, labels, act_lens, label_lens, blank, fastemit_lambda=0.0, workspace=None):
-    """costs [B] (float32) of the RNNT loss on logits = relu(f[:, :, None] + g[:, None]) @ weight.T + bias.
-
-    f [B,T,H], g [B,U,H] (projected encoder / prediction outputs; rounded to bf16 if they are not),
-    weight [V,H] and bias [V] of the joint's last Linear (float32 or bf16), labels [B,U-1] int64,
-    lengths [B] int64.  No gradient is recorded.
-    """
-    _require_gpu(f, "joint_rnnt_forward")
+def _check(f, g, weight, bias):
+    _require_gpu(f, "joint_rnnt_loss")
     if f.dim() != 3 or g.dim() != 3 or f.shape[0] != g.shape[0] or f.shape[2] != g.shape[2]:
         raise ValueError("f must be [B,T,H] and g [B,U,H]")
-    B, T, H = f.shape
-    U = g.shape[1]
-    V = weight.shape[0]
-    if weight.dim() != 2 or weight.shape[1] != H or (bias is not None and bias.shape != (V,)):
+    V, H = weight.shape[0], f.shape[2]
+    if weight.dim() != 2 or weight.shape[1] != H or (bias is not None and tuple(bias.shape) != (V,)):
         raise ValueError("weight must be [V,H] and bias [V]")
-    f = f.detach().to(torch.bfloat16).contiguous()
-    g = g.detach().to(torch.bfloat16).contiguous()
+
+
+def _forward(f16, g16, weight, bias, labels, act_lens, label_lens, blank, fastemit_lambda, workspace):
+    B, T, H = f16.shape
+    U, V = g16.shape[1], weight.shape[0]
+    device = f16.device
     wdtype = torch.float32 if weight.dtype == torch.float32 else torch.bfloat16
     weight = weight.detach().to(wdtype).contiguous()
     bias = None if bias is None else bias.detach().to(wdtype).contiguous()
-    device = f.device
-    if workspace is None:
-        workspace = joint_workspace(B, T, U, H, V, device)
     costs = torch.empty(B, dtype=torch.float32, device=device)
+    tiles = torch.empty(1, dtype=torch.int32, device=device)
     with torch.cuda.device(device):
         status = _native.lib().mi_joint_rnnt_forward(
-            _ptr(f), _ptr(g), _ptr(weight), _ptr(bias),
+            _ptr(f16), _ptr(g16), _ptr(weight), _ptr(bias),
             _native.DTYPE_F32 if wdtype == torch.float32 else _native.DTYPE_BF16, _labels_ptr(labels),
-            _ptr(act_lens), _ptr(label_lens), _ptr(costs), B, T, U, H, V, int(blank), float(fastemit_lambda), 1,
-            _ptr(workspace), workspace.numel(), _stream(device),
+            _ptr(act_lens), _ptr(label_lens), _ptr(costs), _ptr(tiles), B, T, U, H, V, int(blank),
+            float(fastemit_lambda), 1, _ptr(workspace), workspace.numel(), _stream(device),
         )  # fmt: skip
     _native.check_status(status, "joint_rnnt_forward")
-    return costs
+    return costs, tiles
+
+
+def joint_rnnt_forward(f, g, weight, bias, labels, act_lens, label_lens, blank, fastemit_lambda=0.0, workspace=None):
+    """costs [B] (float32) of the RNNT loss on logits = relu(f[:, :, None] + g[:, None]) @ weight.T + bias.
+
+    f [B,T,H], g [B,U,H] (projected encoder / prediction outputs; rounded to bf16 if they are not), weight [V,H] and
+    bias [V] of the joint's last Linear (float32 or bf16), labels [B,U-1] int64, lengths [B] int64.  Nothing is
+    recorded for autograd.
+    """
+    _check(f, g, weight, bias)
+    f16 = f.detach().to(torch.bfloat16).contiguous()
+    g16 = g.detach().to(torch.bfloat16).contiguous()
+    if workspace is None:
+        workspace = joint_workspace(f.shape[0], f.shape[1], g.shape[1], f.shape[2], weight.shape[0], f.device)
+    return _forward(f16, g16, weight, bias, labels, act_lens, label_lens, blank, fastemit_lambda, workspace)[0]
+
+
+class JointRNNTLoss(torch.autograd.Function):
+    """costs [B] = RNNT loss of the ReLU joint's logits, differentiable in f, g, weight, bias."""
+
+    @staticmethod
+    def forward(ctx, f, g, weight, bias, labels, act_lens, label_lens, blank, fastemit_lambda, clamp):
+        _check(f, g, weight, bias)
+        if clamp < 0:
+            raise ValueError("`clamp` must be 0.0 or positive float value.")
+        f16 = f.detach().to(torch.bfloat16).contiguous()
+        g16 = g.detach().to(torch.bfloat16).contiguous()
+        B, T, H = f16.shape
+        workspace = joint_workspace(B, T, g16.shape[1], H, weight.shape[0], f.device)
+        costs, tiles = _forward(f16, g16, weight, bias, labels, act_lens, label_lens, blank, fastemit_lambda, workspace)
+        ctx.save_for_backward(f16, g16, weight, labels, act_lens, label_lens, tiles)
+        ctx.workspace = workspace
+        ctx.has_bias = bias is not None
+        ctx.bias_dtype = None if bias is None else bias.dtype
+        ctx.in_dtypes = (f.dtype, g.dtype)
+        ctx.args = (int(blank), float(fastemit_lambda), float(clamp))
+        return costs
+
+    @staticmethod
+    def backward(ctx, grad_costs):
+        f16, g16, weight, labels, act_lens, label_lens, tiles = ctx.saved_tensors
+        blank, fastemit_lambda, clamp = ctx.args
+        B, T, H = f16.shape
+        U, V = g16.shape[1], weight.shape[0]
+        device = f16.device
+        lib = _native.lib()
+        NP = lib.mi_joint_padded_vocabulary(V)
+        ntiles = int(tiles.item())  # sizes the buffers below: the one host read-back of this op
+        rows = ntiles * 128
+        dlogits = torch.empty(rows, NP, dtype=torch.bfloat16, device=device)
+        row_ft = torch.empty(rows, dtype=torch.int64, device=device)
+        row_gu = torch.empty(rows, dtype=torch.int64, device=device)
+        grad_costs = grad_costs.to(torch.float32)
+        stride = 0 if grad_costs.numel() == 1 else (grad_costs.stride(0) if grad_costs.dim() else 0)
+        with torch.cuda.device(device):
+            status = lib.mi_joint_rnnt_backward_logits(
+                _ptr(f16), _ptr(g16), _labels_ptr(labels), _ptr(act_lens), _ptr(label_lens), _ptr(dlogits),
+                _ptr(row_ft), _ptr(row_gu), ntiles, _ptr(grad_costs), int(stride), 1.0, B, T, U, H, V, blank,
+                fastemit_lambda, clamp, _ptr(ctx.workspace), ctx.workspace.numel(), _stream(device),
+            )  # fmt: skip
+        _native.check_status(status, "joint_rnnt_loss backward")
+        ctx.workspace = None
+        dl = dlogits[:, :V]
+        # hidden activations of the valid cells (zero rows reuse cell 0; their gradient rows are zero)
+        hidden = torch.relu(f16.view(B * T, H).index_select(0, row_ft) + g16.view(B * U, H).index_select(0, row_gu))
+        w16 = weight.to(torch.bfloat16)
+        d_weight = d_bias = d_f = d_g = None
+        if ctx.needs_input_grad[2]:
+            d_weight = (dl.t() @ hidden).to(weight.dtype)
+        if ctx.has_bias and ctx.needs_input_grad[3]:
+            d_bias = dl.float().sum(0).to(ctx.bias_dtype)
+        if ctx.needs_input_grad[0] or ctx.needs_input_grad[1]:
+            d_hidden = (dl @ w16).float() * (hidden > 0)
+            if ctx.needs_input_grad[0]:
+                d_f = torch.zeros(B * T, H, dtype=torch.float32, device=device).index_add_(0, row_ft, d_hidden)
+                d_f = d_f.view(B, T, H).to(ctx.in_dtypes[0])
+            if ctx.needs_input_grad[1]:
+                d_g = torch.zeros(B * U, H, dtype=torch.float32, device=device).index_add_(0, row_gu, d_hidden)
+                d_g = d_g.view(B, U, H).to(ctx.in_dtypes[1])
+        return d_f, d_g, d_weight, d_bias, None, None, None, None, None, None
+
+
+def joint_rnnt_loss(f, g, weight, bias, labels, act_lens, label_lens, blank, fastemit_lambda=0.0, clamp=0.0):
+    """Per-utterance RNNT costs [B] of the joint's logits, with gradients to f, g, weight and bias."""
+    return JointRNNTLoss.apply(f, g, weight, bias, labels, act_lens, label_lens, blank, fastemit_lambda, clamp)
