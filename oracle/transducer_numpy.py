@@ -25,6 +25,9 @@ How each function is pinned (tests/test_oracle_*.py):
                     path, torch autograd of an alpha-only recursion,
                     llForward == beta(0,0) ........................... pinned
   multiblank_* FastEmit  derived only, as for TDT
+  joint_rnnt_loss   torch autograd (float64) through relu, linear and an
+                    alpha-only recursion, with the bf16 roundings applied
+                    straight-through; the loss part is rnnt_loss above  pinned
   rnnt_logprobs*    torch log_softmax + gather (the reference's own etalon,
                     parts/k2/rnnt_logprobs.py:19-48) and torch autograd
                     through it, in float64 ........................... pinned
@@ -626,3 +629,46 @@ def rnnt_logprobs_grad(logits, targets, blank, grad_target_scores, grad_blank_sc
     current = np.take_along_axis(grad, idx, axis=-1)[..., 0]
     np.put_along_axis(grad, idx, np.where(has_target, at_target, current)[..., None], axis=-1)
     return np.where(cell[..., None], grad, 0.0)
+
+
+# ----------------------------------------------------------------------------------------
+# Joint network + loss (nemo/collections/asr/modules/rnnt.py:1707-1724, :1759-1777)
+# ----------------------------------------------------------------------------------------
+def bf16_round(x):
+    """x rounded to the nearest bfloat16 (ties to even), returned as float64."""
+    a = np.ascontiguousarray(x, dtype=np.float32)
+    bits = a.view(np.uint32).astype(np.uint64)
+    rounded = ((bits + 0x7FFF + ((bits >> 16) & 1)) & 0xFFFF0000).astype(np.uint32)
+    out = rounded.view(np.float32).astype(np.float64)
+    return np.where(np.isfinite(a), out, a.astype(np.float64))
+
+
+def joint_rnnt_loss(f, g, weight, bias, labels, act_lens, label_lens, blank, fastemit_lambda=0.0, clamp=0.0, grad_costs=None):
+    """RNNT loss of the ReLU joint's logits under bf16-autocast arithmetic, and its gradients.
+
+    logits[b,t,u,:] = relu(bf16(f[b,t] + g[b,u])) @ bf16(weight).T + bias   (modules/rnnt.py:1707-1724;
+    operands rounded to bf16, products and sums exact here -- float32 accumulation on the GPU; the bias
+    enters as bf16(bias) + bf16(bias - bf16(bias)), i.e. to about 16 bits).  The loss and the gradient of
+    the logits are rnnt_loss's; the gradients of f, g, weight, bias follow by the chain rule with every
+    rounding treated as the identity (what autograd does under autocast).
+    Returns (costs, d_f, d_g, d_weight, d_bias).
+    """
+    f = bf16_round(f)
+    g = bf16_round(g)
+    w = bf16_round(weight)
+    B, T, H = f.shape
+    U, V = g.shape[1], w.shape[0]
+    if bias is None:
+        b_eff = np.zeros(V)
+    else:
+        b_hi = bf16_round(bias)
+        b_eff = b_hi + bf16_round(np.asarray(bias, dtype=np.float32) - b_hi.astype(np.float32))
+    hidden = np.maximum(bf16_round(f[:, :, None, :] + g[:, None, :, :]), 0.0)  # [B,T,U,H]
+    logits = hidden @ w.T + b_eff
+    costs, d_logits, _ = rnnt_loss(logits, labels, act_lens, label_lens, blank, fastemit_lambda, clamp)
+    if grad_costs is not None:
+        d_logits = d_logits * np.asarray(grad_costs, dtype=np.float64).reshape(B, 1, 1, 1)
+    d_weight = np.einsum('btuv,btuh->vh', d_logits, hidden)
+    d_bias = d_logits.sum(axis=(0, 1, 2))
+    d_hidden = (d_logits @ w) * (hidden > 0)
+    return costs, d_hidden.sum(axis=2), d_hidden.sum(axis=1), d_weight, d_bias

@@ -225,3 +225,36 @@ def multiblank_autograd(logits, labels, blank, big_blank_durations, sigma, lam=0
     g_lab = torch.zeros_like(lp) if g_lab is None else g_lab
     lp.backward(g_blank + (1.0 + lam) * g_lab)
     return float(nll.detach()) * (1.0 + lam), x.grad.numpy()
+
+
+def joint_autograd(f, g, weight, bias, labels, blank, grad_costs):
+    """Costs and gradients of sum_b grad_costs[b] * nll_b through relu(f+g) @ W.T + bias, all utterances at
+    full length, by torch autograd in float64; `f`, `g`, `weight`, `bias` must already be exactly
+    representable in bf16, and the rounding of f+g to bf16 is applied straight-through."""
+    f = torch.tensor(np.asarray(f, dtype=np.float64), requires_grad=True)
+    g = torch.tensor(np.asarray(g, dtype=np.float64), requires_grad=True)
+    w = torch.tensor(np.asarray(weight, dtype=np.float64), requires_grad=True)
+    b = torch.tensor(np.asarray(bias, dtype=np.float64), requires_grad=True)
+    s = f[:, :, None, :] + g[:, None, :, :]
+    s = s + (s.detach().float().to(torch.bfloat16).double() - s.detach())
+    logits = torch.nn.functional.linear(torch.relu(s), w, b)
+    B, T, U, _ = logits.shape
+    costs = []
+    for i in range(B):
+        lp = torch.log_softmax(logits[i], dim=-1)
+        alpha = [[None] * U for _ in range(T)]
+        alpha[0][0] = torch.zeros((), dtype=torch.float64)
+        for t in range(T):
+            for u in range(U):
+                if t == 0 and u == 0:
+                    continue
+                terms = []
+                if t > 0:
+                    terms.append(alpha[t - 1][u] + lp[t - 1, u, blank])
+                if u > 0:
+                    terms.append(alpha[t][u - 1] + lp[t, u - 1, labels[i][u - 1]])
+                alpha[t][u] = terms[0] if len(terms) == 1 else _lse(terms[0], terms[1])
+        costs.append(-(alpha[T - 1][U - 1] + lp[T - 1, U - 1, blank]))
+    costs = torch.stack(costs)
+    (costs * torch.tensor(np.asarray(grad_costs, dtype=np.float64))).sum().backward()
+    return costs.detach().numpy(), f.grad.numpy(), g.grad.numpy(), w.grad.numpy(), b.grad.numpy()

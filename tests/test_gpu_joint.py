@@ -1,0 +1,122 @@
+"""GPU parity of the fused joint + RNNT loss (mi_joint_rnnt_forward / mi_joint_rnnt_backward_logits through
+speech_amd.joint) against oracle.joint_rnnt_loss.
+
+Tolerances.  Costs: 1e-5 relative (the bar of the loss itself; float32 accumulation against the oracle's exact
+sums of the same bf16 operands).  Gradients: the kernel stores the gradient of the logits as bf16 and the two GEMMs
+return bf16, as the reference's autocast backward does, so each gradient tensor is held to 2^-7 of its own largest
+entry."""
+
+import numpy as np
+import pytest
+import torch
+
+import oracle
+from speech_amd.joint import joint_rnnt_forward, joint_rnnt_loss
+from speech_amd import RNNTLossNumba
+
+from gpu_utils import DEV
+
+pytestmark = pytest.mark.gpu
+
+
+def make_case(seed, B, T, U, H, V, ragged=True, scale=1.0):
+    rng = np.random.RandomState(seed)
+    f = torch.tensor(rng.randn(B, T, H) * scale, dtype=torch.bfloat16)
+    g = torch.tensor(rng.randn(B, U, H) * scale, dtype=torch.bfloat16)
+    W = torch.tensor(rng.randn(V, H) / np.sqrt(H), dtype=torch.float32)
+    bias = torch.tensor(rng.randn(V) * 0.5, dtype=torch.float32)
+    labels = rng.randint(0, V - 1, size=(B, U - 1))
+    if ragged:
+        al, ll = rng.randint(1, T + 1, size=B), rng.randint(0, U, size=B)
+        al[0], ll[-1] = T, U - 1
+    else:
+        al, ll = np.full(B, T), np.full(B, U - 1)
+    return f, g, W, bias, labels, al, ll
+
+
+def dev_ints(*arrays):
+    return [torch.tensor(np.asarray(a), dtype=torch.int64, device=DEV) for a in arrays]
+
+
+def check(seed, B, T, U, H, V, lam=0.0, clamp=0.0, ragged=True, bias_on=True, weight_dtype=torch.float32):
+    f, g, W, bias, labels, al, ll = make_case(seed, B, T, U, H, V, ragged)
+    rng = np.random.RandomState(seed + 1000)
+    gc = (rng.rand(B) + 0.5).astype(np.float32)
+    Wq = W.to(weight_dtype)
+    bq = bias.to(weight_dtype) if bias_on else None
+    ref = oracle.joint_rnnt_loss(f.float().numpy(), g.float().numpy(), Wq.float().numpy(),
+                                 None if bq is None else bq.float().numpy(), labels, al, ll, V - 1, lam, clamp, gc)  # fmt: skip
+    fd, gd = f.to(DEV).requires_grad_(True), g.to(DEV).requires_grad_(True)
+    Wd = Wq.to(DEV).requires_grad_(True)
+    bd = None if bq is None else bq.to(DEV).requires_grad_(True)
+    lab, ald, lld = dev_ints(labels, al, ll)
+    costs = joint_rnnt_loss(fd, gd, Wd, bd, lab, ald, lld, V - 1, lam, clamp)
+    (costs * torch.tensor(gc, device=DEV)).sum().backward()
+    torch.cuda.synchronize()
+    assert costs.dtype == torch.float32 and costs.shape == (B,)
+    np.testing.assert_allclose(costs.detach().cpu().numpy(), ref[0], rtol=1e-5)
+    got = [fd.grad, gd.grad, Wd.grad] + ([] if bd is None else [bd.grad])
+    for name, x, want in zip(("d_f", "d_g", "d_weight", "d_bias"), got, ref[1:]):
+        assert x.shape == want.shape, name
+        err = np.abs(x.float().cpu().numpy() - want).max()
+        assert err <= 2.0**-7 * np.abs(want).max() + 1e-7, (name, err, np.abs(want).max())
+    assert fd.grad.dtype == torch.bfloat16 and Wd.grad.dtype == weight_dtype
+    return costs
+
+
+@pytest.mark.parametrize("H", [512, 640])
+@pytest.mark.parametrize("V", [2, 37, 128, 129, 1025])
+def test_small_lattices_every_vocabulary_tiling(H, V):
+    check(V + H, 3, 7, 5, H, V)
+
+
+def test_fastemit_and_clamp():
+    check(1, 3, 9, 6, 640, 130, lam=0.01, clamp=0.05)
+
+
+def test_full_lengths_no_bias_bf16_weights():
+    check(2, 2, 6, 4, 640, 300, ragged=False, bias_on=False, weight_dtype=torch.bfloat16)
+
+
+def test_many_tiles_per_utterance_and_tile_tails():
+    # T_b * U_b of 1, 127, 128, 390 and 559 cells: a full tile, tails of 1, 6, 47 and 127 rows
+    f, g, W, bias, labels, _, _ = make_case(3, 5, 130, 13, 640, 257, ragged=False)
+    al, ll = np.array([1, 127, 16, 130, 43]), np.array([0, 0, 7, 2, 12])
+    ref = oracle.joint_rnnt_loss(f.float().numpy(), g.float().numpy(), W.numpy(), bias.numpy(), labels, al, ll, 256)
+    lab, ald, lld = dev_ints(labels, al, ll)
+    fd, gd = f.to(DEV).requires_grad_(True), g.to(DEV).requires_grad_(True)
+    Wd, bd = W.to(DEV).requires_grad_(True), bias.to(DEV).requires_grad_(True)
+    costs = joint_rnnt_loss(fd, gd, Wd, bd, lab, ald, lld, 256)
+    costs.sum().backward()
+    np.testing.assert_allclose(costs.detach().cpu().numpy(), ref[0], rtol=1e-5)
+    for x, want in zip((fd.grad, gd.grad, Wd.grad, bd.grad), ref[1:]):
+        assert np.abs(x.float().cpu().numpy() - want).max() <= 2.0**-7 * np.abs(want).max()
+    # frames and label positions outside an utterance receive exactly nothing
+    for b in range(5):
+        assert torch.all(fd.grad[b, al[b] :] == 0) and torch.all(gd.grad[b, ll[b] + 1 :] == 0)
+
+
+def test_forward_agrees_with_the_loss_on_materialised_logits():
+    """The unfused pipeline of the reference: joint tensor first, then the loss module on it."""
+    f, g, W, bias, labels, al, ll = make_case(4, 4, 30, 11, 640, 1025)
+    al[1], ll[2] = 30, 10
+    lab, ald, lld = dev_ints(labels, al, ll)
+    fd, gd, Wd, bd = f.to(DEV), g.to(DEV), W.to(DEV), bias.to(DEV)
+    fused = joint_rnnt_forward(fd, gd, Wd, bd, lab, ald, lld, 1024)
+    hidden = torch.relu(fd.unsqueeze(2) + gd.unsqueeze(1)).float()
+    logits = hidden @ Wd.to(torch.bfloat16).float().t() + bd
+    unfused = RNNTLossNumba(blank=1024, reduction='none')(logits.contiguous(), lab, ald, lld)
+    np.testing.assert_allclose(fused.cpu().numpy(), unfused.cpu().numpy(), rtol=2e-5)
+
+
+def test_rejects_unsupported_hidden_size_and_bad_shapes():
+    lab, ald, lld = dev_ints(np.zeros((2, 2)), [3, 3], [2, 2])
+    f = torch.zeros(2, 3, 256, dtype=torch.bfloat16, device=DEV)
+    g = torch.zeros(2, 3, 256, dtype=torch.bfloat16, device=DEV)
+    W = torch.zeros(5, 256, device=DEV)
+    with pytest.raises(RuntimeError):
+        joint_rnnt_forward(f, g, W, None, lab, ald, lld, 4)
+    with pytest.raises(ValueError):
+        joint_rnnt_forward(f, g[:, :, :128], W, None, lab, ald, lld, 4)
+    with pytest.raises(RuntimeError):
+        joint_rnnt_forward(f.cpu(), g.cpu(), W.cpu(), None, lab.cpu(), ald.cpu(), lld.cpu(), 4)

@@ -1,0 +1,66 @@
+"""Pins oracle.joint_rnnt_loss (joint network + RNNT loss under bf16-autocast arithmetic).
+
+The reference holds no vector for joint + loss together; its joint is torch's own relu / Linear
+(nemo/collections/asr/modules/rnnt.py:1707-1724, :1759-1777).  So the oracle is checked against those
+library routines and their autograd, in float64, on inputs that are exact in bf16; the loss itself is
+oracle.rnnt_loss, pinned by the reference's golden vectors elsewhere.
+"""
+
+import numpy as np
+import pytest
+import torch
+
+import oracle
+from oracle.transducer_numpy import bf16_round
+
+from helpers import joint_autograd
+
+
+def test_bf16_round_matches_torch():
+    rng = np.random.RandomState(0)
+    x = np.concatenate([rng.randn(4000) * 10.0 ** rng.randint(-6, 6, size=4000), [0.0, -0.0, 1.0, 65280.0, 3.0e38]])
+    # exact ties: halfway between two bf16 neighbours
+    ties = (np.arange(1, 200, dtype=np.uint32) << 16 | 0x8000) + 0x3F800000
+    x = np.concatenate([x.astype(np.float32), ties.view(np.float32)])
+    expect = torch.tensor(x, dtype=torch.float32).to(torch.bfloat16).double().numpy()
+    np.testing.assert_array_equal(bf16_round(x), expect)
+
+
+@pytest.mark.parametrize("shape", [(1, 2, 2, 8, 3), (2, 3, 4, 16, 7), (2, 4, 3, 32, 11)])
+def test_against_torch_autograd(shape):
+    B, T, U, H, V = shape
+    rng = np.random.RandomState(B * 100 + T)
+    f, g = bf16_round(rng.randn(B, T, H)), bf16_round(rng.randn(B, U, H))
+    w = bf16_round(rng.randn(V, H) / np.sqrt(H))
+    bias = bf16_round(rng.randn(V))
+    labels = rng.randint(0, V - 1, size=(B, U - 1))
+    gc = rng.rand(B) + 0.5
+    costs, d_f, d_g, d_w, d_b = oracle.joint_rnnt_loss(f, g, w, bias, labels, [T] * B, [U - 1] * B, V - 1, grad_costs=gc)
+    ref = joint_autograd(f, g, w, bias, labels, V - 1, gc)
+    for got, want in zip((costs, d_f, d_g, d_w, d_b), ref):
+        np.testing.assert_allclose(got, want, rtol=1e-9, atol=1e-11)
+
+
+def test_ragged_lengths_are_the_trimmed_problems():
+    B, T, U, H, V = 3, 5, 4, 16, 9
+    rng = np.random.RandomState(7)
+    f, g = rng.randn(B, T, H), rng.randn(B, U, H)
+    w, bias = rng.randn(V, H) / 4, rng.randn(V)
+    labels = rng.randint(0, V - 1, size=(B, U - 1))
+    al, ll = np.array([5, 2, 4]), np.array([1, 3, 0])
+    costs, d_f, d_g, d_w, d_b = oracle.joint_rnnt_loss(f, g, w, bias, labels, al, ll, V - 1, fastemit_lambda=0.01)
+    sum_w, sum_b = np.zeros_like(d_w), np.zeros_like(d_b)
+    for b in range(B):
+        Tb, Ub = al[b], ll[b] + 1
+        c1, f1, g1, w1, b1 = oracle.joint_rnnt_loss(
+            f[b : b + 1, :Tb], g[b : b + 1, :Ub], w, bias, labels[b : b + 1, : Ub - 1], [Tb], [Ub - 1], V - 1,
+            fastemit_lambda=0.01,
+        )
+        np.testing.assert_allclose(costs[b], c1[0], rtol=1e-12)
+        np.testing.assert_allclose(d_f[b, :Tb], f1[0], atol=1e-12)
+        np.testing.assert_allclose(d_g[b, :Ub], g1[0], atol=1e-12)
+        assert np.all(d_f[b, Tb:] == 0) and np.all(d_g[b, Ub:] == 0)
+        sum_w += w1
+        sum_b += b1
+    np.testing.assert_allclose(d_w, sum_w, atol=1e-11)
+    np.testing.assert_allclose(d_b, sum_b, atol=1e-11)
