@@ -7,9 +7,9 @@ to the loss (:1573-1578); autograd then keeps that tensor and a gradient of the 
   forward   one kernel forms the logits tile by tile on the matrix cores (bf16 operands, float32 accumulation: the
             arithmetic of bf16 autocast) and keeps only each cell's log-softmax denominator and its blank / label
             log-probs; the lattice kernel turns those into the costs;
-  backward  the same kernel recomputes the logits and writes their gradient as bf16, one row per VALID lattice
-            cell (padded cells are never touched); two library GEMMs give d weight and d hidden, and d hidden is
-            summed over u into d f and over t into d g.
+  backward  the same kernel recomputes the logits and writes their gradient and the ReLU outputs as bf16, one row
+            per VALID lattice cell (padded cells are never touched); two library GEMMs give d weight and d hidden,
+            and a reduction kernel sums d hidden over u into d f and over t into d g.
 
 `joint_rnnt_loss` is differentiable in f, g, weight and bias; `joint_rnnt_forward` is the no-grad form.
 Limits: ReLU joint without dropout (the reference's default `jointnet.activation`), H in {512, 640}.
@@ -112,35 +112,49 @@ class JointRNNTLoss(torch.autograd.Function):
         ntiles = int(tiles.item())  # sizes the buffers below: the one host read-back of this op
         rows = ntiles * 128
         dlogits = torch.empty(rows, NP, dtype=torch.bfloat16, device=device)
+        hidden = torch.empty(rows, H, dtype=torch.bfloat16, device=device)
         row_ft = torch.empty(rows, dtype=torch.int64, device=device)
         row_gu = torch.empty(rows, dtype=torch.int64, device=device)
         grad_costs = grad_costs.to(torch.float32)
         stride = 0 if grad_costs.numel() == 1 else (grad_costs.stride(0) if grad_costs.dim() else 0)
+        workspace = ctx.workspace
         with torch.cuda.device(device):
             status = lib.mi_joint_rnnt_backward_logits(
                 _ptr(f16), _ptr(g16), _labels_ptr(labels), _ptr(act_lens), _ptr(label_lens), _ptr(dlogits),
-                _ptr(row_ft), _ptr(row_gu), ntiles, _ptr(grad_costs), int(stride), 1.0, B, T, U, H, V, blank,
-                fastemit_lambda, clamp, _ptr(ctx.workspace), ctx.workspace.numel(), _stream(device),
+                _ptr(hidden), _ptr(row_ft), _ptr(row_gu), ntiles, _ptr(grad_costs), int(stride), 1.0, B, T, U, H, V,
+                blank, fastemit_lambda, clamp, _ptr(workspace), workspace.numel(), _stream(device),
             )  # fmt: skip
         _native.check_status(status, "joint_rnnt_loss backward")
-        ctx.workspace = None
-        dl = dlogits[:, :V]
-        # hidden activations of the valid cells (zero rows reuse cell 0; their gradient rows are zero)
-        hidden = torch.relu(f16.view(B * T, H).index_select(0, row_ft) + g16.view(B * U, H).index_select(0, row_gu))
-        w16 = weight.to(torch.bfloat16)
         d_weight = d_bias = d_f = d_g = None
         if ctx.needs_input_grad[2]:
-            d_weight = (dl.t() @ hidden).to(weight.dtype)
+            # [NP, rows] x [rows, H]: the padded vocabulary rows of dlogits are zero, so are theirs here
+            d_weight = torch.mm(dlogits.t(), hidden)[:V].to(weight.dtype)
         if ctx.has_bias and ctx.needs_input_grad[3]:
-            d_bias = dl.float().sum(0).to(ctx.bias_dtype)
+            d_bias = dlogits.sum(0, dtype=torch.float32)[:V].to(ctx.bias_dtype)
         if ctx.needs_input_grad[0] or ctx.needs_input_grad[1]:
-            d_hidden = (dl @ w16).float() * (hidden > 0)
-            if ctx.needs_input_grad[0]:
-                d_f = torch.zeros(B * T, H, dtype=torch.float32, device=device).index_add_(0, row_ft, d_hidden)
-                d_f = d_f.view(B, T, H).to(ctx.in_dtypes[0])
-            if ctx.needs_input_grad[1]:
-                d_g = torch.zeros(B * U, H, dtype=torch.float32, device=device).index_add_(0, row_gu, d_hidden)
-                d_g = d_g.view(B, U, H).to(ctx.in_dtypes[1])
+            # the forward call's packed weights [NP, H+16] bf16, read in place (their padded rows are zero)
+            packed, prow, pitch = ctypes.c_void_p(), ctypes.c_int(), ctypes.c_int()
+            status = lib.mi_joint_packed_weights(
+                _ptr(workspace), workspace.numel(), B, T, U, H, V, ctypes.byref(packed), ctypes.byref(prow),
+                ctypes.byref(pitch),
+            )  # fmt: skip
+            _native.check_status(status, "joint_rnnt_loss backward")
+            off = packed.value - workspace.data_ptr()
+            w_packed = workspace[off : off + prow.value * pitch.value * 2].view(torch.bfloat16)
+            w_packed = w_packed.view(prow.value, pitch.value)[:, :H]
+            d_hidden = torch.mm(dlogits, w_packed)  # [rows, H] bf16
+            want_f, want_g = ctx.needs_input_grad[0], ctx.needs_input_grad[1]
+            d_f32 = torch.empty(B, T, H, dtype=torch.float32, device=device) if want_f else None
+            d_g32 = torch.empty(B, U, H, dtype=torch.float32, device=device) if want_g else None
+            with torch.cuda.device(device):
+                status = lib.mi_joint_reduce_hidden(
+                    _ptr(d_hidden), _ptr(hidden), _ptr(act_lens), _ptr(label_lens), _ptr(d_f32), _ptr(d_g32), ntiles,
+                    B, T, U, H, V, _ptr(workspace), workspace.numel(), _stream(device),
+                )  # fmt: skip
+            _native.check_status(status, "joint_rnnt_loss backward")
+            d_f = None if d_f32 is None else d_f32.to(ctx.in_dtypes[0])
+            d_g = None if d_g32 is None else d_g32.to(ctx.in_dtypes[1])
+        ctx.workspace = None
         return d_f, d_g, d_weight, d_bias, None, None, None, None, None, None
 
 
