@@ -13,10 +13,13 @@ lengths), inputs already in HBM.  Prints ONE JSON line:
   kernels      mean duration of each pipeline kernel over the timed steps (ms)
   copy_probe   bandwidth a plain device copy reaches on this GPU (GB/s, read + write)
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload 0..5] [--op loss|logprobs] [--no-cpu-baseline]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload 0..5] [--op loss|logprobs|joint] [--no-cpu-baseline]
 
 --op logprobs measures the compact log-prob op on the same tensors instead (speech_amd.k2.rnnt_logprobs
 forward + backward with given upstream gradients; RNNT workloads only).
+--op joint measures the fused joint + loss (speech_amd.joint.joint_rnnt_loss, forward + backward to f, g, weight,
+bias) on joint inputs of the same lattice shape (H = 640, bf16); its roofline is the matrix cores: useful
+flops of the logit recomputation kernel (2 * valid cells * V * H) over its mean duration, against 2.5 PFLOP/s.
 """
 
 import argparse
@@ -47,7 +50,7 @@ def parse_args():
     ap.add_argument("--steps", type=int, default=30)
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--workload", type=int, default=1, help="index into speech_amd.synthetic.CONFIGS (1 = north star)")
-    ap.add_argument("--op", choices=["loss", "logprobs"], default="loss")
+    ap.add_argument("--op", choices=["loss", "logprobs", "joint"], default="loss")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--cpu-sample-utterances", type=int, default=16)
     return ap.parse_args()
@@ -110,6 +113,84 @@ def cpu_baseline_logprobs(cfg, acts, labels, act_lens, label_lens, g_target, g_b
     }  # fmt: skip
 
 
+MFMA_BF16_PEAK_TFLOPS = 2500.0  # MI355X dense bf16, published peak
+JOINT_HIDDEN = 640  # joint_hidden of the reference's FastConformer transducer configs
+
+
+def run_joint(args, torch, dev, cfg, labels, act_lens, label_lens):
+    """--op joint: one step = joint_rnnt_loss forward + backward (gradients of f, g, weight, bias)."""
+    import numpy as np
+
+    from speech_amd import _native
+    from speech_amd.joint import joint_rnnt_loss
+
+    B, T, U, V, H = cfg.B, cfg.T, cfg.U, cfg.V, JOINT_HIDDEN
+    gen = torch.Generator(device=dev).manual_seed(1234)
+    f = torch.randn(B, T, H, device=dev, generator=gen).to(torch.bfloat16).requires_grad_(True)
+    g = torch.randn(B, U, H, device=dev, generator=gen).to(torch.bfloat16).requires_grad_(True)
+    weight = (torch.randn(V, H, device=dev, generator=gen) / H**0.5).requires_grad_(True)
+    bias = (torch.randn(V, device=dev, generator=gen) * 0.1).requires_grad_(True)
+    valid = int((act_lens * (label_lens + 1)).sum())
+
+    def step():
+        for p in (f, g, weight, bias):
+            p.grad = None
+        costs = joint_rnnt_loss(f, g, weight, bias, labels, act_lens, label_lens, cfg.blank, cfg.fastemit_lambda,
+                                max(cfg.clamp, 0.0))  # fmt: skip
+        costs.sum().backward()
+        return costs
+
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+    _native.profile_enable(args.steps, ["denominator_pass", "lattice", "gradient_pass"])
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        costs = step()
+    torch.cuda.synchronize()
+    wall = time.perf_counter() - t0
+    kernels = _native.profile_read()
+    _native.profile_disable()
+    assert bool(torch.isfinite(costs).all()), "non-finite costs"
+    ms_per_step = wall * 1e3 / args.steps
+    grad_ms, grad_n = kernels["gradient_pass"]
+    grad_s = grad_ms * 1e-3 / max(grad_n, 1)
+    flops = 2.0 * valid * V * H
+    achieved = flops / grad_s / 1e12
+    result = {
+        "metric": "fused joint + RNNT loss fwd+bwd: logit elems/s and achieved MFMA TFLOP/s vs peak",
+        "value": cfg.elems / (ms_per_step * 1e-3),
+        "unit": "logit elems/s",
+        "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": ms_per_step,
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
+        "config": {"workload": cfg.name.replace("_f32", "") + "_joint_H%d_bf16" % H, "B": B, "T": T, "U": U, "V": V, "H": H,
+                   "valid_cells": valid, "cells": B * T * U},
+        "roofline": {
+            "kernel": "joint_lse_kernel<H=%d, gradient variant>" % H, "bound": "mfma", "achieved": achieved,
+            "peak": MFMA_BF16_PEAK_TFLOPS, "unit": "TFLOP/s", "frac": achieved / MFMA_BF16_PEAK_TFLOPS,
+            "traffic": None, "algorithmic_flops_per_launch": flops, "avg_launch_ms": grad_s * 1e3, "launches": grad_n,
+        },
+        "kernels": {k: (ms / max(n_, 1)) for k, (ms, n_) in kernels.items() if n_},
+        "whole_job": {"useful_tflop_per_step": 4 * flops / 1e12,
+                      "note": "forward and recomputation kernels plus the two library GEMMs of the backward"},
+    }  # fmt: skip
+    if not args.no_cpu_baseline:
+        import oracle
+
+        Tb, Ub = int(act_lens[0]), int(label_lens[0]) + 1
+        x = (f[:1, :Tb].detach().float().cpu().numpy(), g[:1, :Ub].detach().float().cpu().numpy(),
+             weight.detach().cpu().numpy(), bias.detach().cpu().numpy())  # fmt: skip
+        t0 = time.perf_counter()
+        oracle.joint_rnnt_loss(*x, labels[:1, : Ub - 1].cpu().numpy(), [Tb], [Ub - 1], cfg.blank)
+        dt = time.perf_counter() - t0
+        result["cpu_baseline"] = {
+            "value": Tb * Ub * V / dt, "unit": "logit elems/s", "cores": 1, "kind": "port",
+            "sample": f"utterance 0 of {B} at its own lengths ({Tb} x {Ub} cells), forward + backward, {dt:.2f} s "
+                      "wall (numpy float64; the lattice part in interpreted per-cell loops)",
+        }  # fmt: skip
+    print(json.dumps(result))
+
+
 def main():
     args = parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
@@ -129,6 +210,12 @@ def main():
     _native.lib()  # fail now if the HIP library is missing
 
     cfg, acts, labels, act_lens, label_lens = synthetic.make_inputs(args.workload, device=dev, generate_on_device=True)
+    if args.op == "joint":
+        if cfg.D or cfg.big_blank_durations:
+            print("bench.py: --op joint runs on the RNNT workloads", file=sys.stderr)
+            sys.exit(2)
+        del acts
+        return run_joint(args, torch, dev, cfg, labels, act_lens, label_lens)
     acts.requires_grad_(True)
     if cfg.D:
         loss = TDTLossNumba(blank=cfg.blank, durations=cfg.durations, reduction='none',
