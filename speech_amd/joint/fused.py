@@ -127,8 +127,12 @@ class JointRNNTLoss(torch.autograd.Function):
         _native.check_status(status, "joint_rnnt_loss backward")
         d_weight = d_bias = d_f = d_g = None
         if ctx.needs_input_grad[2]:
-            # [NP, rows] x [rows, H]: the padded vocabulary rows of dlogits are zero, so are theirs here
-            d_weight = torch.mm(dlogits.t(), hidden)[:V].to(weight.dtype)
+            # [NP, rows] x [rows, H], the long axis split 64 ways (rows is a multiple of 128): the library's kernels
+            # for one such product leave most of the GPU idle.  Partial products and their sum are float32.  The
+            # padded vocabulary rows of dlogits are zero, so are theirs here.
+            parts = torch.bmm(dlogits.view(64, rows // 64, NP).transpose(1, 2), hidden.view(64, rows // 64, H),
+                              out_dtype=torch.float32)  # fmt: skip
+            d_weight = parts.sum(0)[:V].to(weight.dtype)
         if ctx.has_bias and ctx.needs_input_grad[3]:
             d_bias = dlogits.sum(0, dtype=torch.float32)[:V].to(ctx.bias_dtype)
         if ctx.needs_input_grad[0] or ctx.needs_input_grad[1]:
