@@ -215,7 +215,8 @@ int mi_joint_rnnt_forward(const void* f, const void* g, const void* weight, cons
 /* Backward of the fused joint, first half: the logits are recomputed tile by tile exactly as in the forward call
  * and turned into their gradient (gpu_rnnt_kernel.py:340-403 with grad_scale folded in, as mi_rnnt_backward), which
  * is stored as bf16 for the two matrix products that finish the job (d weight = dlogits^T . hidden, d hidden =
- * dlogits . weight; `hidden` [rows][H] bf16, the ReLU outputs of the same rows, is written alongside): one row per lattice cell in the kernel's tile order -- utterance by utterance, cell t*U_b + u,
+ * dlogits . weight; `hidden` [rows][H+16] bf16, the ReLU outputs of the same rows followed by 1, 1 and
+ * zeros, is written alongside: column H of dlogits^T . hidden is then the gradient of the bias): one row per lattice cell in the kernel's tile order -- utterance by utterance, cell t*U_b + u,
  * each utterance padded to a multiple of 128 rows with zero rows -- and padded_vocabulary(V) columns, the ones
  * beyond V zero.  row_ft / row_gu receive, per row, the flat indices b*T + t and b*U + u of the cell's rows in f
  * and g (0 for the zero rows).  `tiles` is the number of 128-row tiles the three buffers hold: at least what
@@ -231,7 +232,7 @@ int mi_joint_rnnt_backward_logits(const void* f, const void* g, const int64_t* l
 
 /* Backward of the fused joint, last step: d_hidden [rows][H] bf16 (= dlogits . weight, rows as above) times the
  * ReLU derivative (hidden > 0), summed over u into d_f [B,T,H] and over t into d_g [B,U,H] (float32; either may be
- * NULL; frames and label positions outside an utterance get zeros).  `hidden` [rows][H] bf16 is what
+ * NULL; frames and label positions outside an utterance get zeros).  `hidden` [rows][H+16] bf16 is what
  * mi_joint_rnnt_backward_logits wrote, `tiles` the same count as there; the workspace is the forward call's. */
 int mi_joint_reduce_hidden(const void* d_hidden, const void* hidden, const int64_t* act_lens, const int64_t* label_lens,
                            float* d_f, float* d_g, int tiles, int B, int T, int U, int H, int V, void* workspace,

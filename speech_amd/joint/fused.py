@@ -112,7 +112,7 @@ class JointRNNTLoss(torch.autograd.Function):
         ntiles = int(tiles.item())  # sizes the buffers below: the one host read-back of this op
         rows = ntiles * 128
         dlogits = torch.empty(rows, NP, dtype=torch.bfloat16, device=device)
-        hidden = torch.empty(rows, H, dtype=torch.bfloat16, device=device)
+        hidden = torch.empty(rows, H + 16, dtype=torch.bfloat16, device=device)  # activations, then 1, 1, 0, ...
         row_ft = torch.empty(rows, dtype=torch.int64, device=device)
         row_gu = torch.empty(rows, dtype=torch.int64, device=device)
         grad_costs = grad_costs.to(torch.float32)
@@ -126,15 +126,18 @@ class JointRNNTLoss(torch.autograd.Function):
             )  # fmt: skip
         _native.check_status(status, "joint_rnnt_loss backward")
         d_weight = d_bias = d_f = d_g = None
-        if ctx.needs_input_grad[2]:
-            # [NP, rows] x [rows, H], the long axis split 64 ways (rows is a multiple of 128): the library's kernels
-            # for one such product leave most of the GPU idle.  Partial products and their sum are float32.  The
-            # padded vocabulary rows of dlogits are zero, so are theirs here.
-            parts = torch.bmm(dlogits.view(64, rows // 64, NP).transpose(1, 2), hidden.view(64, rows // 64, H),
+        want_bias = ctx.has_bias and ctx.needs_input_grad[3]
+        if ctx.needs_input_grad[2] or want_bias:
+            # [NP, rows] x [rows, H+16], the long axis split 64 ways (rows is a multiple of 128): the library's kernels
+            # for one such product leave most of the GPU idle.  Partial products and their sum are float32.  Column
+            # H of the result is dlogits summed over the rows, the gradient of the bias (hidden holds ones there).
+            parts = torch.bmm(dlogits.view(64, rows // 64, NP).transpose(1, 2), hidden.view(64, rows // 64, H + 16),
                               out_dtype=torch.float32)  # fmt: skip
-            d_weight = parts.sum(0)[:V].to(weight.dtype)
-        if ctx.has_bias and ctx.needs_input_grad[3]:
-            d_bias = dlogits.sum(0, dtype=torch.float32)[:V].to(ctx.bias_dtype)
+            total = parts.sum(0)
+            if ctx.needs_input_grad[2]:
+                d_weight = total[:V, :H].to(weight.dtype)
+            if want_bias:
+                d_bias = total[:V, H].to(ctx.bias_dtype)
         if ctx.needs_input_grad[0] or ctx.needs_input_grad[1]:
             # the forward call's packed weights [NP, H+16] bf16, read in place (their padded rows are zero)
             packed, prow, pitch = ctypes.c_void_p(), ctypes.c_int(), ctypes.c_int()
