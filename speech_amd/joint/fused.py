@@ -35,13 +35,27 @@ def joint_workspace(B, T, U, H, V, device):
     return torch.empty(nbytes.value, dtype=torch.uint8, device=device)
 
 
-def _check(f, g, weight, bias):
+def _check(f, g, weight, bias, labels, act_lens, label_lens):
+    """Shapes, dtypes and devices (the checks certify_inputs makes for the loss modules, rnnt_pytorch.py:601-634)."""
     _require_gpu(f, "joint_rnnt_loss")
     if f.dim() != 3 or g.dim() != 3 or f.shape[0] != g.shape[0] or f.shape[2] != g.shape[2]:
         raise ValueError("f must be [B,T,H] and g [B,U,H]")
-    V, H = weight.shape[0], f.shape[2]
-    if weight.dim() != 2 or weight.shape[1] != H or (bias is not None and tuple(bias.shape) != (V,)):
-        raise ValueError("weight must be [V,H] and bias [V]")
+    B, U = f.shape[0], g.shape[1]
+    if weight.dim() != 2 or weight.shape[1] != f.shape[2]:
+        raise ValueError("weight must be [V,H]")
+    if bias is not None and tuple(bias.shape) != (weight.shape[0],):
+        raise ValueError("bias must be [V]")
+    for name, t, shape in (("labels", labels, (B, U - 1)), ("act_lens", act_lens, (B,)), ("label_lens", label_lens, (B,))):
+        if t.dtype != torch.int64:
+            raise TypeError(f"{name} must be int64")
+        if tuple(t.shape) != shape:
+            raise ValueError(f"{name} must have shape {list(shape)}, got {list(t.shape)}")
+        if not t.is_contiguous():
+            raise ValueError(f"{name} must be contiguous")
+    for name, t in (("g", g), ("weight", weight), ("bias", bias), ("labels", labels), ("act_lens", act_lens),
+                    ("label_lens", label_lens)):  # fmt: skip
+        if t is not None and t.device != f.device:
+            raise ValueError(f"{name} must be on {f.device}")
 
 
 def _forward(f16, g16, weight, bias, labels, act_lens, label_lens, blank, fastemit_lambda, workspace):
@@ -71,7 +85,7 @@ def joint_rnnt_forward(f, g, weight, bias, labels, act_lens, label_lens, blank, 
     bias [V] of the joint's last Linear (float32 or bf16), labels [B,U-1] int64, lengths [B] int64.  Nothing is
     recorded for autograd.
     """
-    _check(f, g, weight, bias)
+    _check(f, g, weight, bias, labels, act_lens, label_lens)
     f16 = f.detach().to(torch.bfloat16).contiguous()
     g16 = g.detach().to(torch.bfloat16).contiguous()
     if workspace is None:
@@ -84,7 +98,7 @@ class JointRNNTLoss(torch.autograd.Function):
 
     @staticmethod
     def forward(ctx, f, g, weight, bias, labels, act_lens, label_lens, blank, fastemit_lambda, clamp):
-        _check(f, g, weight, bias)
+        _check(f, g, weight, bias, labels, act_lens, label_lens)
         if clamp < 0:
             raise ValueError("`clamp` must be 0.0 or positive float value.")
         f16 = f.detach().to(torch.bfloat16).contiguous()

@@ -120,3 +120,14 @@ def test_rejects_unsupported_hidden_size_and_bad_shapes():
         joint_rnnt_forward(f, g[:, :, :128], W, None, lab, ald, lld, 4)
     with pytest.raises(RuntimeError):
         joint_rnnt_forward(f.cpu(), g.cpu(), W.cpu(), None, lab.cpu(), ald.cpu(), lld.cpu(), 4)
+    with pytest.raises(TypeError):
+        joint_rnnt_forward(f, g, W, None, lab, ald.int(), lld, 4)
+    with pytest.raises(ValueError):
+        joint_rnnt_forward(f, g, W, None, lab[:, :1], ald, lld, 4)
+    with pytest.raises(ValueError):
+        joint_rnnt_forward(f, g, W, None, lab, ald.cpu(), lld, 4)
+
+
+def test_many_utterances():
+    """More utterances than a workgroup scans linearly: the tile -> utterance search must land on the right one."""
+    check(5, 70, 3, 2, 512, 19)
