@@ -231,12 +231,13 @@ int mi_joint_rnnt_backward_logits(const void* f, const void* g, const int64_t* l
                                   void* stream);
 
 /* Backward of the fused joint, last step: d_hidden [rows][H] bf16 (= dlogits . weight, rows as above) times the
- * ReLU derivative (hidden > 0), summed over u into d_f [B,T,H] and over t into d_g [B,U,H] (float32; either may be
- * NULL; frames and label positions outside an utterance get zeros).  `hidden` [rows][H+16] bf16 is what
- * mi_joint_rnnt_backward_logits wrote, `tiles` the same count as there; the workspace is the forward call's. */
-int mi_joint_reduce_hidden(const void* d_hidden, const void* hidden, const int64_t* act_lens, const int64_t* label_lens,
-                           float* d_f, float* d_g, int tiles, int B, int T, int U, int H, int V, void* workspace,
-                           size_t workspace_bytes, void* stream);
+ * ReLU derivative, summed over u into d_f [B,T,H] and over t into d_g [B,U,H] (float32; either may be NULL; frames
+ * and label positions outside an utterance get zeros).  The derivative is recomputed from f and g (the forward
+ * call's bf16 inputs), `tiles` is the same count as in mi_joint_rnnt_backward_logits, the workspace the forward
+ * call's. */
+int mi_joint_reduce_hidden(const void* d_hidden, const void* f, const void* g, const int64_t* act_lens,
+                           const int64_t* label_lens, float* d_f, float* d_g, int tiles, int B, int T, int U, int H,
+                           int V, void* workspace, size_t workspace_bytes, void* stream);
 
 /* Where the forward call left the packed weights inside its workspace: *rows x *pitch bf16, row n = weight[n, :]
  * followed by the bias columns (rows beyond V are zero in the first H columns), so that the d_hidden product can

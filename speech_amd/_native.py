@@ -84,7 +84,7 @@ _SIGNATURES = {
     "mi_joint_rnnt_backward_logits": [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _c_int, _vp, _c_int, _c_float,
                                       _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_float, _c_float, _vp,
                                       _c_size_t, _vp],
-    "mi_joint_reduce_hidden": [_vp, _vp, _vp, _vp, _vp, _vp, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _vp,
+    "mi_joint_reduce_hidden": [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _vp,
                                _c_size_t, _vp],
     "mi_joint_packed_weights": [_vp, _c_size_t, _c_int, _c_int, _c_int, _c_int, _c_int, ctypes.POINTER(_vp),
                                 ctypes.POINTER(_c_int), ctypes.POINTER(_c_int)],

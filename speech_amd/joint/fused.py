@@ -169,7 +169,7 @@ class JointRNNTLoss(torch.autograd.Function):
             d_g32 = torch.empty(B, U, H, dtype=torch.float32, device=device) if want_g else None
             with torch.cuda.device(device):
                 status = lib.mi_joint_reduce_hidden(
-                    _ptr(d_hidden), _ptr(hidden), _ptr(act_lens), _ptr(label_lens), _ptr(d_f32), _ptr(d_g32), ntiles,
+                    _ptr(d_hidden), _ptr(f16), _ptr(g16), _ptr(act_lens), _ptr(label_lens), _ptr(d_f32), _ptr(d_g32), ntiles,
                     B, T, U, H, V, _ptr(workspace), workspace.numel(), _stream(device),
                 )  # fmt: skip
             _native.check_status(status, "joint_rnnt_loss backward")
