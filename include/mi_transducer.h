@@ -199,18 +199,25 @@ int mi_rnnt_logprobs_backward(const void* logits, int act_dtype, const int64_t* 
 /* ---- joint projection fused into the forward pass --------------------------------------
  * Replaces RNNTJoint.joint_after_projection followed by the loss forward
  * (nemo/collections/asr/modules/rnnt.py:1707-1724 and :1573-1578) for the default joint network
- * (ReLU, no dropout, Linear(H -> V); :1759-1777): the [B,T,U,V] tensor is never written.
+ * (ReLU, optional Dropout, Linear(H -> V); :1759-1777): the [B,T,U,V] tensor is never written.
  *   f [B,T,H], g [B,U,H]: bf16, the projected encoder / prediction-network outputs (16-byte aligned);
  *   weight [V,H], bias [V] (nullable): float32 or bf16 (weight_dtype), the final Linear layer;
  *   logits = relu(f[b,t] + g[b,u]) . weight^T + bias with bf16 operands and float32 accumulation
  *   (what the reference computes under bf16 autocast, minus its rounding of the logits to bf16).
  * costs[b] as mi_rnnt_forward; the workspace (mi_joint_workspace_bytes) ends up holding the same
- * lattice state.  H must be 512 or 640; V any. */
+ * lattice state.  H must be 512 or 640; V any.
+ * Dropout of the hidden activations (the joint network's Dropout(p) between activation and Linear, :1772-1776):
+ * dropout_p in [0, 1), 0 = none.  The keep mask is a pure function of (dropout_seed, cell, hidden unit): the
+ * backward calls below must be given the same two values and then see the same mask; kept activations are scaled
+ * by 1 / (1 - p).  mi_joint_dropout_mask writes that mask ([B*T*U][H] bytes, 1 = kept) for tests. */
 int mi_joint_workspace_bytes(int B, int T, int U, int H, int V, size_t* out_bytes);
 int mi_joint_rnnt_forward(const void* f, const void* g, const void* weight, const void* bias, int weight_dtype,
                           const int64_t* labels, const int64_t* act_lens, const int64_t* label_lens, float* costs,
-                          int* tile_count, int B, int T, int U, int H, int V, int blank, float fastemit_lambda,
-                          int with_betas, void* workspace, size_t workspace_bytes, void* stream);
+                          int* tile_count, float dropout_p, unsigned long long dropout_seed, int B, int T, int U, int H,
+                          int V, int blank, float fastemit_lambda, int with_betas, void* workspace,
+                          size_t workspace_bytes, void* stream);
+int mi_joint_dropout_mask(unsigned char* mask, float dropout_p, unsigned long long dropout_seed, int B, int T, int U,
+                          int H, void* stream);
 
 /* Backward of the fused joint, first half: the logits are recomputed tile by tile exactly as in the forward call
  * and turned into their gradient (gpu_rnnt_kernel.py:340-403 with grad_scale folded in, as mi_rnnt_backward), which
@@ -226,9 +233,9 @@ int mi_joint_padded_vocabulary(int V);
 int mi_joint_rnnt_backward_logits(const void* f, const void* g, const int64_t* labels, const int64_t* act_lens,
                                   const int64_t* label_lens, void* dlogits, void* hidden, int64_t* row_ft,
                                   int64_t* row_gu, int tiles, const float* grad_scale, int grad_scale_stride,
-                                  float grad_mul, int B, int T, int U, int H, int V, int blank,
-                                  float fastemit_lambda, float clamp, void* workspace, size_t workspace_bytes,
-                                  void* stream);
+                                  float grad_mul, float dropout_p, unsigned long long dropout_seed, int B, int T, int U,
+                                  int H, int V, int blank, float fastemit_lambda, float clamp, void* workspace,
+                                  size_t workspace_bytes, void* stream);
 
 /* Backward of the fused joint, last step: d_hidden [rows][H] bf16 (= dlogits . weight, rows as above) times the
  * ReLU derivative, summed over u into d_f [B,T,H] and over t into d_g [B,U,H] (float32; either may be NULL; frames
@@ -236,8 +243,9 @@ int mi_joint_rnnt_backward_logits(const void* f, const void* g, const int64_t* l
  * call's bf16 inputs), `tiles` is the same count as in mi_joint_rnnt_backward_logits, the workspace the forward
  * call's. */
 int mi_joint_reduce_hidden(const void* d_hidden, const void* f, const void* g, const int64_t* act_lens,
-                           const int64_t* label_lens, float* d_f, float* d_g, int tiles, int B, int T, int U, int H,
-                           int V, void* workspace, size_t workspace_bytes, void* stream);
+                           const int64_t* label_lens, float* d_f, float* d_g, int tiles, float dropout_p,
+                           unsigned long long dropout_seed, int B, int T, int U, int H, int V, void* workspace,
+                           size_t workspace_bytes, void* stream);
 
 /* Where the forward call left the packed weights inside its workspace: *rows x *pitch bf16, row n = weight[n, :]
  * followed by the bias columns (rows beyond V are zero in the first H columns), so that the d_hidden product can

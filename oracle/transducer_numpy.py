@@ -643,14 +643,17 @@ def bf16_round(x):
     return np.where(np.isfinite(a), out, a.astype(np.float64))
 
 
-def joint_rnnt_loss(f, g, weight, bias, labels, act_lens, label_lens, blank, fastemit_lambda=0.0, clamp=0.0, grad_costs=None):
+def joint_rnnt_loss(f, g, weight, bias, labels, act_lens, label_lens, blank, fastemit_lambda=0.0, clamp=0.0, grad_costs=None,
+                    keep_mask=None, dropout_p=0.0):
     """RNNT loss of the ReLU joint's logits under bf16-autocast arithmetic, and its gradients.
 
-    logits[b,t,u,:] = relu(bf16(f[b,t] + g[b,u])) @ bf16(weight).T + bias   (modules/rnnt.py:1707-1724;
-    operands rounded to bf16, products and sums exact here -- float32 accumulation on the GPU; the bias
-    enters as bf16(bias) + bf16(bias - bf16(bias)), i.e. to about 16 bits).  The loss and the gradient of
-    the logits are rnnt_loss's; the gradients of f, g, weight, bias follow by the chain rule with every
-    rounding treated as the identity (what autograd does under autocast).
+    logits[b,t,u,:] = drop(relu(bf16(f[b,t] + g[b,u]))) @ bf16(weight).T + bias   (modules/rnnt.py:1707-1724,
+    joint_net = ReLU, Dropout, Linear :1766-1777; operands rounded to bf16, products and sums exact here --
+    float32 accumulation on the GPU; the bias enters as bf16(bias) + bf16(bias - bf16(bias)), i.e. to about
+    16 bits).  drop(x) = bf16(x * keep_mask / (1 - dropout_p)) for a given boolean keep_mask [B,T,U,H]
+    (torch.nn.functional.dropout's definition; which units are kept is the caller's business), identity without
+    one.  The loss and the gradient of the logits are rnnt_loss's; the gradients of f, g, weight, bias follow by the
+    chain rule with every rounding treated as the identity (what autograd does under autocast).
     Returns (costs, d_f, d_g, d_weight, d_bias).
     """
     f = bf16_round(f)
@@ -663,12 +666,19 @@ def joint_rnnt_loss(f, g, weight, bias, labels, act_lens, label_lens, blank, fas
     else:
         b_hi = bf16_round(bias)
         b_eff = b_hi + bf16_round(np.asarray(bias, dtype=np.float32) - b_hi.astype(np.float32))
-    hidden = np.maximum(bf16_round(f[:, :, None, :] + g[:, None, :, :]), 0.0)  # [B,T,U,H]
+    pre = bf16_round(f[:, :, None, :] + g[:, None, :, :])  # [B,T,U,H]
+    hidden = np.maximum(pre, 0.0)
+    chain = (pre > 0).astype(np.float64)  # d hidden / d pre
+    if keep_mask is not None:
+        scale = np.float32(1.0) / (np.float32(1.0) - np.float32(dropout_p))
+        keep = np.asarray(keep_mask, dtype=bool)
+        hidden = np.where(keep, bf16_round(hidden.astype(np.float32) * scale), 0.0)
+        chain = chain * keep * np.float64(scale)
     logits = hidden @ w.T + b_eff
     costs, d_logits, _ = rnnt_loss(logits, labels, act_lens, label_lens, blank, fastemit_lambda, clamp)
     if grad_costs is not None:
         d_logits = d_logits * np.asarray(grad_costs, dtype=np.float64).reshape(B, 1, 1, 1)
     d_weight = np.einsum('btuv,btuh->vh', d_logits, hidden)
     d_bias = d_logits.sum(axis=(0, 1, 2))
-    d_hidden = (d_logits @ w) * (hidden > 0)
-    return costs, d_hidden.sum(axis=2), d_hidden.sum(axis=1), d_weight, d_bias
+    d_pre = (d_logits @ w) * chain
+    return costs, d_pre.sum(axis=2), d_pre.sum(axis=1), d_weight, d_bias

@@ -227,7 +227,7 @@ def multiblank_autograd(logits, labels, blank, big_blank_durations, sigma, lam=0
     return float(nll.detach()) * (1.0 + lam), x.grad.numpy()
 
 
-def joint_autograd(f, g, weight, bias, labels, blank, grad_costs):
+def joint_autograd(f, g, weight, bias, labels, blank, grad_costs, keep_mask=None, dropout_p=0.0):
     """Costs and gradients of sum_b grad_costs[b] * nll_b through relu(f+g) @ W.T + bias, all utterances at
     full length, by torch autograd in float64; `f`, `g`, `weight`, `bias` must already be exactly
     representable in bf16, and the rounding of f+g to bf16 is applied straight-through."""
@@ -237,7 +237,15 @@ def joint_autograd(f, g, weight, bias, labels, blank, grad_costs):
     b = torch.tensor(np.asarray(bias, dtype=np.float64), requires_grad=True)
     s = f[:, :, None, :] + g[:, None, :, :]
     s = s + (s.detach().float().to(torch.bfloat16).double() - s.detach())
-    logits = torch.nn.functional.linear(torch.relu(s), w, b)
+    hidden = torch.relu(s)
+    if keep_mask is not None:  # dropout with a given mask; its bf16 output rounding is straight-through as well
+        scale = float(np.float32(1.0) / (np.float32(1.0) - np.float32(dropout_p)))
+        hidden = hidden * torch.tensor(np.asarray(keep_mask, dtype=np.float64)) * scale
+        # the product is formed in float32 before the rounding, as on the GPU
+        exact32 = (torch.relu(s).detach().float() * np.float32(scale)).to(torch.bfloat16).double()
+        rounded = torch.where(torch.tensor(np.asarray(keep_mask, dtype=bool)), exact32, torch.zeros_like(exact32))
+        hidden = hidden + (rounded - hidden.detach())
+    logits = torch.nn.functional.linear(hidden, w, b)
     B, T, U, _ = logits.shape
     costs = []
     for i in range(B):

@@ -11,7 +11,7 @@ import pytest
 import torch
 
 import oracle
-from speech_amd.joint import joint_rnnt_forward, joint_rnnt_loss
+from speech_amd.joint import joint_dropout_mask, joint_rnnt_forward, joint_rnnt_loss
 from speech_amd import RNNTLossNumba
 
 from gpu_utils import DEV
@@ -131,3 +131,61 @@ def test_rejects_unsupported_hidden_size_and_bad_shapes():
 def test_many_utterances():
     """More utterances than a workgroup scans linearly: the tile -> utterance search must land on the right one."""
     check(5, 70, 3, 2, 512, 19)
+
+
+@pytest.mark.parametrize("p", [0.2, 0.5])
+def test_dropout_mask_is_a_function_of_the_seed_and_keeps_the_right_share(p):
+    a = joint_dropout_mask(3, 11, 7, 640, p, 1234, DEV)
+    b = joint_dropout_mask(3, 11, 7, 640, p, 1234, DEV)
+    c = joint_dropout_mask(3, 11, 7, 640, p, 1235, DEV)
+    assert torch.equal(a, b) and not torch.equal(a, c)
+    n = a.numel()
+    kept = a.float().mean().item()
+    assert abs(kept - (1 - p)) < 5 * (p * (1 - p) / n) ** 0.5 + 1e-4
+    # no structure along any axis: every frame, label position and hidden unit keeps about the same share
+    for dim in ((0, 2, 3), (0, 1, 3), (0, 1, 2)):
+        share = a.float().mean(dim=dim)
+        m = n / share.numel()
+        assert (share - (1 - p)).abs().max().item() < 6 * (p * (1 - p) / m) ** 0.5
+    # two seeds agree on about p^2 + (1-p)^2 of the units
+    agree = (a == c).float().mean().item()
+    assert abs(agree - (p * p + (1 - p) * (1 - p))) < 0.01
+    assert joint_dropout_mask(2, 3, 4, 512, 0.0, 7, DEV).all()
+
+
+@pytest.mark.parametrize("H,p", [(640, 0.2), (512, 0.5)])
+def test_dropout_parity_with_the_exported_mask(H, p):
+    B, T, U, V = 3, 9, 6, 130
+    f, g, W, bias, labels, al, ll = make_case(21, B, T, U, H, V)
+    seed = 987654321012345
+    keep = joint_dropout_mask(B, T, U, H, p, seed, DEV).cpu().numpy()
+    gc = (np.random.RandomState(3).rand(B) + 0.5).astype(np.float32)
+    ref = oracle.joint_rnnt_loss(f.float().numpy(), g.float().numpy(), W.numpy(), bias.numpy(), labels, al, ll, V - 1,
+                                 0.01, 0.0, gc, keep_mask=keep, dropout_p=p)  # fmt: skip
+    fd, gd = f.to(DEV).requires_grad_(True), g.to(DEV).requires_grad_(True)
+    Wd, bd = W.to(DEV).requires_grad_(True), bias.to(DEV).requires_grad_(True)
+    lab, ald, lld = dev_ints(labels, al, ll)
+    costs = joint_rnnt_loss(fd, gd, Wd, bd, lab, ald, lld, V - 1, 0.01, 0.0, dropout=p, seed=seed)
+    (costs * torch.tensor(gc, device=DEV)).sum().backward()
+    np.testing.assert_allclose(costs.detach().cpu().numpy(), ref[0], rtol=1e-5)
+    for name, x, want in zip(("d_f", "d_g", "d_weight", "d_bias"), (fd.grad, gd.grad, Wd.grad, bd.grad), ref[1:]):
+        err = np.abs(x.float().cpu().numpy() - want).max()
+        assert err <= 2.0**-7 * np.abs(want).max() + 1e-7, (name, err)
+    # the no-grad form sees the same mask; another seed gives other costs
+    again = joint_rnnt_forward(fd, gd, Wd, bd, lab, ald, lld, V - 1, 0.01, dropout=p, seed=seed)
+    other = joint_rnnt_forward(fd, gd, Wd, bd, lab, ald, lld, V - 1, 0.01, dropout=p, seed=seed + 1)
+    assert torch.equal(again, costs.detach()) and not torch.equal(other, costs.detach())
+
+
+def test_dropout_seed_follows_torch_manual_seed():
+    f, g, W, bias, labels, al, ll = make_case(22, 2, 5, 4, 512, 40)
+    lab, ald, lld = dev_ints(labels, al, ll)
+    args = (f.to(DEV), g.to(DEV), W.to(DEV), bias.to(DEV), lab, ald, lld, 39)
+    torch.manual_seed(5)
+    a = joint_rnnt_forward(*args, dropout=0.3)
+    b = joint_rnnt_forward(*args, dropout=0.3)
+    torch.manual_seed(5)
+    c = joint_rnnt_forward(*args, dropout=0.3)
+    assert torch.equal(a, c) and not torch.equal(a, b)
+    with pytest.raises(ValueError):
+        joint_rnnt_forward(*args, dropout=1.0)

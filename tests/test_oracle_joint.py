@@ -64,3 +64,23 @@ def test_ragged_lengths_are_the_trimmed_problems():
         sum_b += b1
     np.testing.assert_allclose(d_w, sum_w, atol=1e-11)
     np.testing.assert_allclose(d_b, sum_b, atol=1e-11)
+
+
+def test_dropout_against_torch_autograd():
+    B, T, U, H, V = 2, 3, 3, 16, 7
+    rng = np.random.RandomState(9)
+    f, g = bf16_round(rng.randn(B, T, H)), bf16_round(rng.randn(B, U, H))
+    w, bias = bf16_round(rng.randn(V, H) / 4), bf16_round(rng.randn(V))
+    labels = rng.randint(0, V - 1, size=(B, U - 1))
+    keep = rng.rand(B, T, U, H) >= 0.3
+    gc = rng.rand(B) + 0.5
+    got = oracle.joint_rnnt_loss(f, g, w, bias, labels, [T] * B, [U - 1] * B, V - 1, grad_costs=gc, keep_mask=keep, dropout_p=0.3)
+    ref = joint_autograd(f, g, w, bias, labels, V - 1, gc, keep_mask=keep, dropout_p=0.3)
+    for a, b in zip(got, ref):
+        np.testing.assert_allclose(a, b, rtol=1e-9, atol=1e-11)
+    # a mask of ones with p = 0 is no dropout at all
+    plain = oracle.joint_rnnt_loss(f, g, w, bias, labels, [T] * B, [U - 1] * B, V - 1, grad_costs=gc)
+    ones = oracle.joint_rnnt_loss(f, g, w, bias, labels, [T] * B, [U - 1] * B, V - 1, grad_costs=gc,
+                                  keep_mask=np.ones((B, T, U, H), dtype=bool), dropout_p=0.0)  # fmt: skip
+    for a, b in zip(plain, ones):
+        np.testing.assert_array_equal(a, b)
