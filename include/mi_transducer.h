@@ -205,7 +205,7 @@ int mi_rnnt_logprobs_backward(const void* logits, int act_dtype, const int64_t* 
  *   logits = relu(f[b,t] + g[b,u]) . weight^T + bias with bf16 operands and float32 accumulation
  *   (what the reference computes under bf16 autocast, minus its rounding of the logits to bf16).
  * costs[b] as mi_rnnt_forward; the workspace (mi_joint_workspace_bytes) ends up holding the same
- * lattice state.  H must be 512 or 640; V any.
+ * lattice state.  H must be one of 256, 320, 384, 512, 640; V any.
  * Dropout of the hidden activations (the joint network's Dropout(p) between activation and Linear, :1772-1776):
  * dropout_p in [0, 1), 0 = none.  The keep mask is a pure function of (dropout_seed, cell, hidden unit): the
  * backward calls below must be given the same two values and then see the same mask; kept activations are scaled

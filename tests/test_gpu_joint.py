@@ -3,8 +3,8 @@ speech_amd.joint) against oracle.joint_rnnt_loss.
 
 Tolerances.  Costs: 1e-5 relative (the bar of the loss itself; float32 accumulation against the oracle's exact
 sums of the same bf16 operands).  Gradients: the kernel stores the gradient of the logits as bf16 and the two GEMMs
-return bf16, as the reference's autocast backward does, so each gradient tensor is held to 2^-7 of its own largest
-entry."""
+return bf16, as the reference's autocast backward does (two roundings of 2^-9 each on every term of the sums over u
+and t, whose terms may cancel), so each gradient tensor is held to 2^-6 of its own largest entry."""
 
 import numpy as np
 import pytest
@@ -59,12 +59,12 @@ def check(seed, B, T, U, H, V, lam=0.0, clamp=0.0, ragged=True, bias_on=True, we
     for name, x, want in zip(("d_f", "d_g", "d_weight", "d_bias"), got, ref[1:]):
         assert x.shape == want.shape, name
         err = np.abs(x.float().cpu().numpy() - want).max()
-        assert err <= 2.0**-7 * np.abs(want).max() + 1e-7, (name, err, np.abs(want).max())
+        assert err <= 2.0**-6 * np.abs(want).max() + 1e-7, (name, err, np.abs(want).max())
     assert fd.grad.dtype == torch.bfloat16 and Wd.grad.dtype == weight_dtype
     return costs
 
 
-@pytest.mark.parametrize("H", [512, 640])
+@pytest.mark.parametrize("H", [256, 320, 384, 512, 640])
 @pytest.mark.parametrize("V", [2, 37, 128, 129, 1025])
 def test_small_lattices_every_vocabulary_tiling(H, V):
     check(V + H, 3, 7, 5, H, V)
@@ -90,7 +90,7 @@ def test_many_tiles_per_utterance_and_tile_tails():
     costs.sum().backward()
     np.testing.assert_allclose(costs.detach().cpu().numpy(), ref[0], rtol=1e-5)
     for x, want in zip((fd.grad, gd.grad, Wd.grad, bd.grad), ref[1:]):
-        assert np.abs(x.float().cpu().numpy() - want).max() <= 2.0**-7 * np.abs(want).max()
+        assert np.abs(x.float().cpu().numpy() - want).max() <= 2.0**-6 * np.abs(want).max()
     # frames and label positions outside an utterance receive exactly nothing
     for b in range(5):
         assert torch.all(fd.grad[b, al[b] :] == 0) and torch.all(gd.grad[b, ll[b] + 1 :] == 0)
@@ -111,13 +111,13 @@ def test_forward_agrees_with_the_loss_on_materialised_logits():
 
 def test_rejects_unsupported_hidden_size_and_bad_shapes():
     lab, ald, lld = dev_ints(np.zeros((2, 2)), [3, 3], [2, 2])
-    f = torch.zeros(2, 3, 256, dtype=torch.bfloat16, device=DEV)
-    g = torch.zeros(2, 3, 256, dtype=torch.bfloat16, device=DEV)
-    W = torch.zeros(5, 256, device=DEV)
+    f = torch.zeros(2, 3, 192, dtype=torch.bfloat16, device=DEV)
+    g = torch.zeros(2, 3, 192, dtype=torch.bfloat16, device=DEV)
+    W = torch.zeros(5, 192, device=DEV)
     with pytest.raises(RuntimeError):
         joint_rnnt_forward(f, g, W, None, lab, ald, lld, 4)
     with pytest.raises(ValueError):
-        joint_rnnt_forward(f, g[:, :, :128], W, None, lab, ald, lld, 4)
+        joint_rnnt_forward(f, g[:, :, :64], W, None, lab, ald, lld, 4)
     with pytest.raises(RuntimeError):
         joint_rnnt_forward(f.cpu(), g.cpu(), W.cpu(), None, lab.cpu(), ald.cpu(), lld.cpu(), 4)
     with pytest.raises(TypeError):
@@ -170,7 +170,7 @@ def test_dropout_parity_with_the_exported_mask(H, p):
     np.testing.assert_allclose(costs.detach().cpu().numpy(), ref[0], rtol=1e-5)
     for name, x, want in zip(("d_f", "d_g", "d_weight", "d_bias"), (fd.grad, gd.grad, Wd.grad, bd.grad), ref[1:]):
         err = np.abs(x.float().cpu().numpy() - want).max()
-        assert err <= 2.0**-7 * np.abs(want).max() + 1e-7, (name, err)
+        assert err <= 2.0**-6 * np.abs(want).max() + 1e-7, (name, err)
     # the no-grad form sees the same mask; another seed gives other costs
     again = joint_rnnt_forward(fd, gd, Wd, bd, lab, ald, lld, V - 1, 0.01, dropout=p, seed=seed)
     other = joint_rnnt_forward(fd, gd, Wd, bd, lab, ald, lld, V - 1, 0.01, dropout=p, seed=seed + 1)
