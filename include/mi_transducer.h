@@ -220,19 +220,20 @@ int mi_joint_dropout_mask(unsigned char* mask, float dropout_p, unsigned long lo
                           int H, void* stream);
 
 /* Backward of the fused joint, first half: the logits are recomputed tile by tile exactly as in the forward call
- * and turned into their gradient (gpu_rnnt_kernel.py:340-403 with grad_scale folded in, as mi_rnnt_backward), which
- * is stored as bf16 for the two matrix products that finish the job (d weight = dlogits^T . hidden, d hidden =
- * dlogits . weight; `hidden` [rows][H+16] bf16, the ReLU outputs of the same rows followed by 1, 1 and
- * zeros, is written alongside: column H of dlogits^T . hidden is then the gradient of the bias): one row per lattice cell in the kernel's tile order -- utterance by utterance, cell t*U_b + u,
- * each utterance padded to a multiple of 128 rows with zero rows -- and padded_vocabulary(V) columns, the ones
- * beyond V zero.  row_ft / row_gu receive, per row, the flat indices b*T + t and b*U + u of the cell's rows in f
- * and g (0 for the zero rows).  `tiles` is the number of 128-row tiles the three buffers hold: at least what
- * mi_joint_rnnt_forward wrote to tile_count (device int32, nullable there), whose workspace this call needs
- * unchanged (forward with with_betas != 0). */
+ * (same dropout_p and dropout_seed) and turned into their gradient (gpu_rnnt_kernel.py:340-403 with grad_scale
+ * folded in, as mi_rnnt_backward), which is stored as bf16 for the two matrix products that finish the job:
+ *   d weight = dlogits^T . hidden   and   d hidden = dlogits . weight.
+ * dlogits [rows][padded_vocabulary(V)] bf16: one row per lattice cell in the kernel's tile order -- utterance by
+ *   utterance, cell t*U_b + u, each utterance padded to a multiple of 128 rows with zero rows; columns beyond V zero.
+ * hidden [rows][H+16] bf16: the joint's hidden activations of the same rows (after ReLU and dropout) followed by
+ *   1, 1 and zeros, so that column H of dlogits^T . hidden is the gradient of the bias.
+ * `tiles` is the number of 128-row tiles the two buffers hold: at least what mi_joint_rnnt_forward wrote to
+ * tile_count (device int32, nullable there), whose workspace this call needs unchanged (forward with
+ * with_betas != 0). */
 int mi_joint_padded_vocabulary(int V);
 int mi_joint_rnnt_backward_logits(const void* f, const void* g, const int64_t* labels, const int64_t* act_lens,
-                                  const int64_t* label_lens, void* dlogits, void* hidden, int64_t* row_ft,
-                                  int64_t* row_gu, int tiles, const float* grad_scale, int grad_scale_stride,
+                                  const int64_t* label_lens, void* dlogits, void* hidden, int tiles,
+                                  const float* grad_scale, int grad_scale_stride,
                                   float grad_mul, float dropout_p, unsigned long long dropout_seed, int B, int T, int U,
                                   int H, int V, int blank, float fastemit_lambda, float clamp, void* workspace,
                                   size_t workspace_bytes, void* stream);

@@ -16,7 +16,7 @@ INCLUDE_DIR = os.path.join(os.path.dirname(_HERE), "include")
 LIB_PATH = os.environ.get("MI_TRANSDUCER_LIB") or os.path.join(CSRC_DIR, "libmi_transducer.so")
 SOURCES = [os.path.join(CSRC_DIR, "mi_transducer.hip")]
 
-ABI_VERSION = 10
+ABI_VERSION = 11
 SUCCESS, INVALID_VALUE, LAUNCH_FAILURE = 0, 1, 2
 DTYPE_F32, DTYPE_BF16, DTYPE_F16 = 0, 1, 2
 
@@ -82,7 +82,7 @@ _SIGNATURES = {
                               _c_int, _c_int, _c_int, _c_int, _c_int, _c_float, _c_int, _vp, _c_size_t, _vp],
     "mi_joint_dropout_mask": [_vp, _c_float, ctypes.c_uint64, _c_int, _c_int, _c_int, _c_int, _vp],
     "mi_joint_padded_vocabulary": [_c_int],
-    "mi_joint_rnnt_backward_logits": [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _c_int, _vp, _c_int, _c_float,
+    "mi_joint_rnnt_backward_logits": [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _c_int, _vp, _c_int, _c_float,
                                       _c_float, ctypes.c_uint64, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int,
                                       _c_float, _c_float, _vp, _c_size_t, _vp],
     "mi_joint_reduce_hidden": [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _c_int, _c_float, ctypes.c_uint64, _c_int, _c_int,

@@ -2873,7 +2873,7 @@ int run_multiblank_fixup(const Common& c, void* grads, const MbParams& prm) {
 
 extern "C" {
 
-int mi_transducer_abi_version(void) { return 10; }
+int mi_transducer_abi_version(void) { return 11; }
 
 int mi_transducer_workspace_bytes(int B, int T, int U, int D, size_t* out_bytes) {
   Layout L;
