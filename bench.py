@@ -52,6 +52,7 @@ def parse_args():
     ap.add_argument("--workload", type=int, default=1, help="index into speech_amd.synthetic.CONFIGS (1 = north star)")
     ap.add_argument("--op", choices=["loss", "logprobs", "joint"], default="loss")
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-graph", action="store_true", help="skip the HIP-graph replay timing of the same step")
     ap.add_argument("--cpu-sample-utterances", type=int, default=16)
     return ap.parse_args()
 
@@ -111,6 +112,59 @@ def cpu_baseline_logprobs(cfg, acts, labels, act_lens, label_lens, g_target, g_b
         "sample": f"first {n_utt} of {cfg.B} utterances of the same batch, full T x U x V, forward + backward, "
                   f"{dt:.2f} s wall (numpy, float64)",
     }  # fmt: skip
+
+
+def graph_replay(torch, cfg, acts, labels, act_lens, label_lens, steps):
+    """The same forward + backward at the function-level seam (caller-owned costs / grads / workspace, grad_output
+    = ones), captured once into a HIP graph and replayed: what a training loop with static shapes pays per step
+    when launch gaps and the Python/autograd layer are out of the picture.  Reported beside the headline, not as it."""
+    from speech_amd.rnnt_loss import rnnt
+
+    B = cfg.B
+    costs = torch.empty(B, dtype=torch.float32, device=acts.device)
+    grads = torch.empty_like(acts)
+    ones = torch.ones(B, dtype=torch.float32, device=acts.device)
+    lam, clamp = cfg.fastemit_lambda, max(cfg.clamp, 0.0)
+    if cfg.D:
+        ws = rnnt.new_workspace(acts, cfg.D)
+
+        def run():
+            rnnt.tdt_forward(acts, labels, act_lens, label_lens, costs, cfg.blank, cfg.durations, lam, cfg.sigma, False,
+                             True, ws)  # fmt: skip
+            rnnt.tdt_backward(acts, labels, act_lens, label_lens, grads, ones, cfg.blank, cfg.durations, lam, clamp,
+                              cfg.sigma, False, ws)  # fmt: skip
+    elif cfg.big_blank_durations:
+        ws = rnnt.new_workspace(acts, len(cfg.big_blank_durations))
+
+        def run():
+            rnnt.multiblank_forward(acts, labels, act_lens, label_lens, costs, cfg.blank, cfg.big_blank_durations, lam,
+                                    cfg.sigma, True, ws)  # fmt: skip
+            rnnt.multiblank_backward(acts, labels, act_lens, label_lens, grads, ones, cfg.blank,
+                                     cfg.big_blank_durations, lam, clamp, cfg.sigma, ws)  # fmt: skip
+    else:
+        ws = rnnt.new_workspace(acts)
+
+        def run():
+            rnnt.rnnt_forward(acts, labels, act_lens, label_lens, costs, cfg.blank, lam, True, ws)
+            rnnt.rnnt_backward(acts, labels, act_lens, label_lens, grads, ones, cfg.blank, lam, clamp, ws)
+
+    run()
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        run()
+    for _ in range(3):
+        graph.replay()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        graph.replay()
+    torch.cuda.synchronize()
+    ms = (time.perf_counter() - t0) * 1e3 / steps
+    assert bool(torch.isfinite(costs).all())
+    del grads
+    return {"ms_per_step": ms, "logit_elems_per_s": cfg.elems / (ms * 1e-3),
+            "what": "mi_*_forward + mi_*_backward (grad_output = 1) replayed from one captured HIP graph"}  # fmt: skip
 
 
 MFMA_BF16_PEAK_TFLOPS = 2500.0  # MI355X dense bf16, published peak
@@ -357,6 +411,8 @@ def main():
         "plan": plan,
         "copy_probe_GBps": copy_gbps,
     }  # fmt: skip
+    if not args.no_graph and not logprobs:
+        result["graph_replay"] = graph_replay(torch, cfg, acts.detach(), labels, act_lens, label_lens, args.steps)
     if not args.no_cpu_baseline and logprobs:
         result["cpu_baseline"] = cpu_baseline_logprobs(
             cfg, acts.detach(), labels, act_lens, label_lens, g_target, g_blank, min(args.cpu_sample_utterances, 8)
