@@ -916,9 +916,11 @@ __global__ __launch_bounds__(512) void tdt_lattice_pair_kernel(
     const int plane0 = lab ? D * Us : 0;
     const bool half_on = !lab || u > 0;  // column 0 has no label arc coming in
     const int seed = half_on ? 1 : 0;    // the emit and the no-emit accumulator are each seeded once
-    double final_arc[D];
+    // arc i lands on this cell from diagonal n on where t = n - u >= its duration: one compare against the
+    // (wave-uniform) diagonal number per arc
+    int nmin[D];
 #pragma unroll
-    for (int i = 0; i < D; ++i) final_arc[i] = -INFINITY;
+    for (int i = 0; i < D; ++i) nmin[i] = half_on ? u + thr[i] : (1 << 29);
     auto step_fn = [&](int n, const float* w) {
       const int t = n - u;
       double x[D];
@@ -926,7 +928,7 @@ __global__ __launch_bounds__(512) void tdt_lattice_pair_kernel(
       for (int i = 0; i < D; ++i) {
         double v = ring[off[i] + plane0 + i * Us + col];
         asm("" : "+v"(v));  // read here, not under the test below
-        x[i] = (half_on && t >= thr[i]) ? v : -INFINITY;
+        x[i] = n >= nmin[i] ? v : -INFINITY;
       }
       const double interior = lse_pair(x, seed);
       // row 0: only a duration-0 label arc gets there (:941-955); its score sits in the label half
@@ -939,9 +941,7 @@ __global__ __launch_bounds__(512) void tdt_lattice_pair_kernel(
       double* slot = ring + cur_off + plane0 + u;
 #pragma unroll
       for (int i = 0; i < D; ++i) {
-        const double ob = wt + (double)w[1 + i];
-        slot[i * Us] = ob;
-        final_arc[i] = (!lab && dur[i] > 0 && u == Ub - 1 && t >= 0 && t + dur[i] == Tb) ? ob : final_arc[i];  // :1040-1071
+        slot[i * Us] = wt + (double)w[1 + i];
       }
 #pragma unroll
       for (int i = 0; i < D; ++i) off[i] = off[i] + slot_stride == ring_len ? 0 : off[i] + slot_stride;
@@ -965,11 +965,20 @@ __global__ __launch_bounds__(512) void tdt_lattice_pair_kernel(
       step_fn(n0, w[0]);
     }
     if (!lab && u == Ub - 1) {
-      // a longer duration ends the utterance from an earlier diagonal: summed in that order
+      // the blank arcs that end the utterance (:1040-1071) leave from cells (Tb - d_i, Ub-1) of this thread's own
+      // column: their alphas are re-read (this thread stored them) and the arc scores formed as in the loop.  A
+      // longer duration ends the utterance from an earlier diagonal: summed in that order.
       double ll_acc = NEG;
 #pragma unroll
-      for (int i = D - 1; i >= 0; --i)
-        if (final_arc[i] != -INFINITY) ll_acc = lse_h(ll_acc, final_arc[i]);
+      for (int i = D - 1; i >= 0; --i) {
+        const int t0 = Tb - dur[i];
+        if (dur[i] > 0 && t0 >= 0) {
+          const float* rp = arcs_b + (size_t)(t0 + u) * row_pitch;
+          const double a = out[(size_t)(t0 + u) * Us];
+          const double wt = (a + (double)rp[0]) - sigma;
+          ll_acc = lse_h(ll_acc, wt + (double)rp[(size_t)(2 + i) * Us]);
+        }
+      }
       ll[2 * b] = ll_acc;
       costs[b] = -(float)ll_acc * cost_scale;
     }
@@ -977,8 +986,19 @@ __global__ __launch_bounds__(512) void tdt_lattice_pair_kernel(
     const int ring_len = R * Us;
     for (int i = threadIdx.x; i < ring_len; i += 2 * Us) ring[i] = NEG;
     __syncthreads();
+    // a blank that ends the utterance (t + d == Tb in the last column, :1137-1148, :1160-1176) is an arc into a
+    // virtual cell beta(Tb, Ub-1) = 0 on diagonal nd: with that cell in the ring it needs no case of its own
+    if (threadIdx.x == 0) ring[(nd % R) * Us + Ub - 1] = 0.0;
+    __syncthreads();
     double* out = betas + (size_t)b * ND * Us + u;
     double last = NEG;
+    // arc i leaves this cell while t + d_i < Tb (<= Tb for the blank arcs of the last column), i.e. on diagonals
+    // n < nmax[i]: one compare against the (wave-uniform) diagonal number per arc.  A blank of duration 0 never
+    // passes (thr = 2^28), a label arc needs a next column.
+    int nmax[D];
+#pragma unroll
+    for (int i = 0; i < D; ++i)
+      nmax[i] = (!lab || u + 1 < Ub) ? Tb + u - thr[i] + ((!lab && u == Ub - 1) ? 1 : 0) : -(1 << 29);
     // ring offsets of the diagonals this half reads: n + d_i (blank arcs, same column) or n + d_i + 1
     // (label arcs, column u+1); both go back by one slot per step
     int off[D];
@@ -995,10 +1015,7 @@ __global__ __launch_bounds__(512) void tdt_lattice_pair_kernel(
         double v = ring[off[i] + col];
         asm("" : "+v"(v));
         const double arc = (tok + (double)w[1 + i]) - sigma;
-        const int d = thr[i];  // blank half: duration 0 never passes
-        const bool reach = t + d < Tb && (!lab || u + 1 < Ub);
-        const bool ends = !lab && t + d == Tb && u == Ub - 1;  // a blank that ends the utterance
-        x[i] = reach ? v + arc : (ends ? arc : -INFINITY);
+        x[i] = n < nmax[i] ? v + arc : -INFINITY;
       }
       // one seed for the no-emit (blank) accumulator, one for the emit accumulator unless it is the last column
       const double interior = lse_pair(x, (!lab || u != Ub - 1) ? 1 : 0);
