@@ -1440,12 +1440,7 @@ __global__ __launch_bounds__(MAXT) void multiblank_lattice_kernel(
     for (int j = 0; j < NJ; ++j) off_in[j] = j - 1 < NB ? ((R - dur[j] % R) % R) * slot_stride : 0;
     int cur_off = 0;
     const int um1 = u > 0 ? u - 1 : 0;
-    // arcs that end the utterance (column Ub-1, t + dur_j == Tb), kept as they pass; gpu_rnnt_kernel.py:548-568
-    double final_arc[NJ];
-#pragma unroll
-    for (int j = 0; j < NJ; ++j) final_arc[j] = NINF;
     auto step_fn = [&](int n, const float* w) {
-      const int t = n - u;
       double x[1 + NJ];
       x[0] = u > 0 ? ring[off_in[0] + um1] : NINF;  // label arc out of (t, u-1)
 #pragma unroll
@@ -1459,7 +1454,6 @@ __global__ __launch_bounds__(MAXT) void multiblank_lattice_kernel(
       for (int j = 0; j < NJ; ++j) {
         const double ob = (a + (double)w[j == 0 ? 0 : 1 + j]) - sigma;
         slot[(1 + j) * Us] = ob + unused[j];
-        final_arc[j] = (u == Ub - 1 && t >= 0 && t + dur[j] == Tb) ? ob : final_arc[j];
       }
 #pragma unroll
       for (int j = 0; j < NJ; ++j) off_in[j] = off_in[j] + slot_stride == ring_len ? 0 : off_in[j] + slot_stride;
@@ -1483,10 +1477,20 @@ __global__ __launch_bounds__(MAXT) void multiblank_lattice_kernel(
       step_fn(n0, w[0]);
     }
     if (u == Ub - 1) {
-      // the standard blank first, then the big blanks in their order (gpu_rnnt_kernel.py:548-568)
-      double acc = final_arc[0];
+      // the blank arcs that end the utterance leave from cells (Tb - dur_j, Ub-1) of this thread's own column
+      // (gpu_rnnt_kernel.py:548-568): their alphas are re-read (this thread stored them) and the arc scores
+      // formed as in the loop -- the standard blank first, then the big blanks in their order
+      double acc = NINF;
 #pragma unroll
-      for (int j = 1; j < NJ; ++j) acc = lse_h(acc, final_arc[j]);
+      for (int j = 0; j < NJ; ++j) {
+        const int t0 = Tb - dur[j];
+        if (t0 >= 0) {  // (unused slots have a duration beyond any utterance)
+          const float* rp = arcs_b + (size_t)(t0 + u) * row_pitch;
+          const double a = out[(size_t)(t0 + u) * Us];
+          const double ob = (a + (double)finite_arc(rp[(size_t)plane[j] * Us])) - sigma;
+          acc = j == 0 ? ob : lse_h(acc, ob);
+        }
+      }
       ll[2 * b] = acc;
       costs[b] = -(float)acc * cost_scale;
     }
@@ -1494,8 +1498,19 @@ __global__ __launch_bounds__(MAXT) void multiblank_lattice_kernel(
     const int ring_len = R * Us;
     for (int i = u; i < ring_len; i += Us) ring[i] = NINF;
     __syncthreads();
+    // a big blank that ends the utterance from column Ub-1 (t + dur == Tb, gpu_rnnt_kernel.py:660-670; the standard
+    // blank does so through the corner cell) is an arc into a virtual cell beta(Tb, Ub-1) = 0 on diagonal nd: with
+    // that cell in the ring it needs no case of its own
+    if (u == 0) ring[(nd % R) * Us + Ub - 1] = 0.0;
+    __syncthreads();
     double* out = betas + (size_t)b * ND * Us + u;
     double last = NINF;
+    // blank arc j leaves this cell while t + dur_j < Tb (<= Tb for a big blank in the last column), the label arc
+    // while t < Tb: diagonals n < nmax, one compare against the (wave-uniform) diagonal number per arc
+    int nmax[NJ];
+#pragma unroll
+    for (int j = 0; j < NJ; ++j) nmax[j] = Tb + u - dur[j] + ((j > 0 && u == Ub - 1) ? 1 : 0);
+    const int nmax_label = u < Ub - 1 ? Tb + u : -(1 << 29);
     // ring offsets of the diagonals n+dur_j; the label arc reads diagonal n+1 like the standard blank
     int off_in[NJ];
 #pragma unroll
@@ -1505,15 +1520,12 @@ __global__ __launch_bounds__(MAXT) void multiblank_lattice_kernel(
     auto step_fn = [&](int n, const float* w) {
       const int t = n - u;
       double x[1 + NJ];
-      x[0] = (t < Tb && u < Ub - 1) ? (ring[off_in[0] + up1] + (double)w[1]) - sigma : NINF;  // label arc to (t, u+1)
+      x[0] = n < nmax_label ? (ring[off_in[0] + up1] + (double)w[1]) - sigma : NINF;  // label arc to (t, u+1)
 #pragma unroll
       for (int j = 0; j < NJ; ++j) {
         const double arc = (double)w[j == 0 ? 0 : 1 + j] - sigma;
-        // a big blank may end the utterance from column Ub-1 (gpu_rnnt_kernel.py:660-670; the standard
-        // blank does so through the corner cell); selects, not branches
         const double via = ring[off_in[j] + u] + arc;
-        const bool ends = j > 0 && t + dur[j] == Tb && u == Ub - 1 && dur[j] != 1;
-        x[1 + j] = t + dur[j] < Tb ? via : (ends ? arc : NINF);
+        x[1 + j] = n < nmax[j] ? via : NINF;  // selects, not branches
       }
       double v = lse_all(x);
       if (t == Tb - 1 && u == Ub - 1) v = (double)w[0] - sigma;  // the corner: one standard blank
