@@ -732,7 +732,9 @@ __global__ __launch_bounds__(64) void tdt_lattice_kernel(const float* __restrict
     for (int i = lane; i < 2 * R * Us; i += 64) ring[i] = kTdtNeg;
     __syncthreads();
     double* out = alphas + (size_t)b * ND * Us;
-    double ll_acc = kTdtNeg;
+    // scores of the blank arcs that end the utterance, one per duration (summed after the loop in the reference's order)
+    double end_term[MI_TRANSDUCER_MAX_DURATIONS];
+    for (int i = 0; i < MI_TRANSDUCER_MAX_DURATIONS; ++i) end_term[i] = -INFINITY;
     for (int n = 0; n < nd; ++n) {
       const int slot = (n % R) * Us;
       const float* rp = arcs_b + (size_t)n * A * Us;
@@ -761,7 +763,7 @@ __global__ __launch_bounds__(64) void tdt_lattice_kernel(const float* __restrict
                 double* q = ne_ring + ((n + d) % R) * Us + u;
                 *q = lse_h(*q, c);
               } else if (t + d == Tb && u == Ub - 1) {
-                ll_acc = lse_h(ll_acc, c);
+                end_term[i] = c;
               }
             }
             if (u + 1 < Ub && t + d < Tb) {
@@ -770,6 +772,12 @@ __global__ __launch_bounds__(64) void tdt_lattice_kernel(const float* __restrict
             }
           }
           if (n == nd - 1) {  // (Tb-1, Ub-1): the last contribution to llForward is in
+            // :1046-1071: the duration-1 term is assigned over the -10000 the sum starts from, longer ones are added
+            double ll_acc = kTdtNeg;
+            for (int i = 0; i < D; ++i) {
+              if (prm.dur[i] == 1) ll_acc = end_term[i];
+              else if (prm.dur[i] > 1 && end_term[i] != -INFINITY) ll_acc = lse_h(ll_acc, end_term[i]);
+            }
             ll[2 * b] = ll_acc;
             costs[b] = -(float)ll_acc * cost_scale;
           }
@@ -966,17 +974,20 @@ __global__ __launch_bounds__(512) void tdt_lattice_pair_kernel(
     }
     if (!lab && u == Ub - 1) {
       // the blank arcs that end the utterance (:1040-1071) leave from cells (Tb - d_i, Ub-1) of this thread's own
-      // column: their alphas are re-read (this thread stored them) and the arc scores formed as in the loop.  A
-      // longer duration ends the utterance from an earlier diagonal: summed in that order.
+      // column: their alphas are re-read (this thread stored them) and the arc scores formed as in the loop.
+      // In the reference's order (:1046-1071): the duration-1 term is ASSIGNED (the -10000 the sum starts from is
+      // gone by then: duration 1 sits at position 0 or 1, and a duration 0 before it is skipped), the longer
+      // durations are added while they fit the utterance.  The difference to a sum seeded with -10000 shows only
+      // when no alignment exists and the terms themselves are down at the sentinel.
       double ll_acc = NEG;
 #pragma unroll
-      for (int i = D - 1; i >= 0; --i) {
+      for (int i = 0; i < D; ++i) {
         const int t0 = Tb - dur[i];
         if (dur[i] > 0 && t0 >= 0) {
           const float* rp = arcs_b + (size_t)(t0 + u) * row_pitch;
           const double a = out[(size_t)(t0 + u) * Us];
-          const double wt = (a + (double)rp[0]) - sigma;
-          ll_acc = lse_h(ll_acc, wt + (double)rp[(size_t)(2 + i) * Us]);
+          const double term = ((a + (double)rp[0]) - sigma) + (double)rp[(size_t)(2 + i) * Us];
+          ll_acc = dur[i] == 1 ? term : lse_h(ll_acc, term);
         }
       }
       ll[2 * b] = ll_acc;

@@ -118,3 +118,26 @@ def test_costs_follow_the_dtype_of_acts_and_cpu_raises_value_error():
         fn(acts.cpu().float(), lab.cpu(), al.cpu(), ll.cpu())
     with pytest.raises(RuntimeError):
         TDTLossNumba(blank=4, durations=[0, 2, 3], reduction='none')(acts, lab, al, ll)  # no duration 1
+
+
+@pytest.mark.parametrize("durations", [[1, 2], [1, 3], [1, 2, 4], [0, 1, 2]])
+def test_utterances_without_an_alignment_follow_the_sentinel_arithmetic(durations):
+    """Without a duration 0 every label needs a frame of its own: more labels than frames leave no alignment, and the
+    reference's result is what its -10000 sentinels add up to (cost about 10000 plus a few arc log-probs).  The
+    forward log-likelihood then shows how the final sum is formed -- the duration-1 term is assigned, not added to
+    the -10000 it starts from (gpu_rnnt_kernel.py:1046-1071) -- so these costs pin that detail.  With duration 0 in
+    the set the same shapes are ordinary cases."""
+    rng = np.random.RandomState(len(durations) * 7 + durations[-1])
+    B, T, U, V = 4, 6, 9, 12
+    D = len(durations)
+    acts = rng.randn(B, T, U, V + D)
+    labels = rng.randint(0, V - 1, size=(B, U - 1))
+    act_lens = np.array([6, 2, 3, 1])
+    label_lens = np.array([8, 5, 3, 4])
+    fn = TDTLossNumba(blank=V - 1, durations=durations, reduction='none', sigma=0.05)
+    costs, grads = call_loss(fn, acts, labels, act_lens, label_lens)
+    c_ref, g_ref, _ = oracle.tdt_loss(acts.astype(np.float32), labels, act_lens, label_lens, V - 1, durations, 0.05)
+    if durations[0] != 0:
+        assert np.all(c_ref > 9000)
+    np.testing.assert_allclose(costs, c_ref, rtol=2e-6)
+    assert np.abs(grads - g_ref).max() <= 1e-5 * max(1.0, np.abs(g_ref).max())
