@@ -355,7 +355,7 @@ def main():
     from speech_amd.rnnt_loss import rnnt, rnnt_pytorch
 
     plan = _native.describe_plan(rnnt._dtype_code(acts), cfg.B, cfg.T, cfg.U, cfg.V, cfg.D,
-                                 max(cfg.durations) if cfg.D else 0,
+                                 max(cfg.durations) if cfg.D else max(cfg.big_blank_durations, default=0),
                                  num_big_blanks=len(cfg.big_blank_durations))  # fmt: skip
 
     grad_ms, grad_n = kernels["gradient_pass"]

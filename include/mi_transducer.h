@@ -292,7 +292,7 @@ int mi_transducer_profile_disable(void);
 /* Which kernels a call with this shape would launch, as text:
  * "denominators=...; lattice=...; cells=...; gradient=..." ("cells=-" when the gradient pass derives
  * its coefficients itself).  D = 0 for RNNT; for TDT pass the largest duration; for the multi-blank
- * loss D = 0 and num_big_blanks > 0 (V counting the big blanks).  Assumes a gradient
+ * loss D = 0, num_big_blanks > 0 (V counting the big blanks) and max_duration the longest big blank.  Assumes a gradient
  * buffer at the 16-byte phase of the logits.  Launches nothing.  For benchmarks, profiles and tests
  * that want to name (or pin) the kernel family a shape maps to. */
 int mi_transducer_describe_plan(int act_dtype, int B, int T, int U, int V, int D, int max_duration,

@@ -1568,6 +1568,93 @@ __global__ __launch_bounds__(MAXT) void multiblank_lattice_kernel(
   }
 }
 
+// Multi-blank lattice for shapes whose ring of arc scores does not fit LDS (a long label axis with long or many big
+// blanks): the same recursion, one thread per column and one barrier per anti-diagonal, but every value is pulled
+// from the alphas / betas this workgroup has already stored in global memory, read back from L2 with device-scope
+// loads.  A step costs an L2 round trip instead of an LDS one -- the price of having a path at all for these shapes.
+// The arithmetic (arc score = (alpha + arc) - sigma, one log-sum-exp over label arc, standard blank, big blanks in
+// their order) is that of multiblank_lattice_kernel, so the two give the same values.
+__global__ __launch_bounds__(1024) void multiblank_lattice_pull_kernel(
+    const float* __restrict__ arcs, double* alphas, double* betas, double* __restrict__ ll, float* __restrict__ costs,
+    const int64_t* __restrict__ act_lens, const int64_t* __restrict__ label_lens, int T, int U, int ND, int Us, int A,
+    float cost_scale, int with_betas, MbParams prm) {
+  const int b = with_betas ? (int)(blockIdx.x >> 1) : (int)blockIdx.x;
+  const int dir = with_betas ? (int)(blockIdx.x & 1) : 0;
+  const int u = threadIdx.x;  // blockDim.x == Us
+  const int Tb = clampi(act_lens[b], 1, T);
+  const int Ub = clampi(label_lens[b] + 1, 1, U);
+  const int nd = Tb + Ub - 1;
+  const int NB = prm.NB;
+  const double sigma = (double)prm.sigma;
+  const double NINF = kLogZero;
+  const size_t row_pitch = (size_t)A * Us;
+  const float* arcs_b = arcs + (size_t)b * ND * row_pitch;
+  auto arc = [&](int n, int plane, int col) { return (double)finite_arc(arcs_b[(size_t)n * row_pitch + (size_t)plane * Us + col]); };
+  auto ld = [&](const double* p) { return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT); };
+  auto st = [&](double* p, double v) { __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT); };
+  // log-sum-exp of x[0..n) in index order; "log 0" entries vanish
+  auto lse_n = [&](const double* x, int n) {
+    double m = x[0];
+    for (int i = 1; i < n; ++i) m = fmax(m, x[i]);
+    float s = 0.f;
+    for (int i = 0; i < n; ++i) s += fast_exp2((float)(x[i] - m) * kLog2e);
+    return m + (double)(__builtin_amdgcn_logf(s) * 0.6931471805599453f);
+  };
+  double x[2 + MI_TRANSDUCER_MAX_BIG_BLANKS];
+  if (dir == 0) {
+    double* out = alphas + (size_t)b * ND * Us;
+    for (int n = 0; n < nd; ++n) {
+      const int t = n - u;
+      if (t >= 0 && t < Tb && u < Ub) {
+        x[0] = u > 0 ? (ld(out + (size_t)(n - 1) * Us + u - 1) + arc(n - 1, 1, u - 1)) - sigma : NINF;
+        x[1] = t >= 1 ? (ld(out + (size_t)(n - 1) * Us + u) + arc(n - 1, 0, u)) - sigma : NINF;
+        for (int i = 0; i < NB; ++i) {
+          const int d = prm.dur[i];
+          x[2 + i] = t >= d ? (ld(out + (size_t)(n - d) * Us + u) + arc(n - d, 2 + i, u)) - sigma : NINF;
+        }
+        double a = lse_n(x, 2 + NB);
+        if (n == 0) a = 0.0;  // (t, u) = (0, 0)
+        st(out + (size_t)n * Us + u, a);
+      }
+      __syncthreads();
+    }
+    if (u == Ub - 1) {
+      // the blank arcs that end the utterance (gpu_rnnt_kernel.py:548-568): the standard blank, then the big blanks
+      double acc = (ld(out + (size_t)(Tb - 1 + u) * Us + u) + arc(Tb - 1 + u, 0, u)) - sigma;
+      for (int i = 0; i < NB; ++i) {
+        const int t0 = Tb - prm.dur[i];
+        if (t0 >= 0) acc = lse_h(acc, (ld(out + (size_t)(t0 + u) * Us + u) + arc(t0 + u, 2 + i, u)) - sigma);
+      }
+      ll[2 * b] = acc;
+      costs[b] = -(float)acc * cost_scale;
+    }
+  } else {
+    double* out = betas + (size_t)b * ND * Us;
+    for (int n = nd - 1; n >= 0; --n) {
+      const int t = n - u;
+      if (t >= 0 && t < Tb && u < Ub) {
+        double v;
+        if (t == Tb - 1 && u == Ub - 1) {
+          v = arc(n, 0, u) - sigma;  // the corner: one standard blank
+        } else {
+          x[0] = u < Ub - 1 ? (ld(out + (size_t)(n + 1) * Us + u + 1) + arc(n, 1, u)) - sigma : NINF;
+          x[1] = t + 1 < Tb ? ld(out + (size_t)(n + 1) * Us + u) + (arc(n, 0, u) - sigma) : NINF;
+          for (int i = 0; i < NB; ++i) {
+            const int d = prm.dur[i];
+            const double a = arc(n, 2 + i, u) - sigma;
+            // a big blank may end the utterance from the last column (gpu_rnnt_kernel.py:660-670)
+            x[2 + i] = t + d < Tb ? ld(out + (size_t)(n + d) * Us + u) + a : ((t + d == Tb && u == Ub - 1) ? 0.0 + a : NINF);
+          }
+          v = lse_n(x, 2 + NB);
+        }
+        st(out + (size_t)n * Us + u, v);
+      }
+      __syncthreads();
+    }
+    if (u == 0) ll[2 * b + 1] = ld(out);  // beta(0,0)
+  }
+}
+
 // Per-cell coefficients of the multi-blank gradient (gpu_rnnt_kernel.py:727-885): the record of the
 // RNNT/TDT cell kernels, plus in out[kCoefBase + i] the FINISHED gradient entry of big blank i
 // (clamped and scaled), which multiblank_fixup_kernel stores over what the gradient pass put there.
@@ -2686,8 +2773,12 @@ int run_tdt_lattice(const Common& c, float* costs, float lambda, int with_betas,
   }
   // general fallback (many durations or a very wide label axis): one wave per lattice
   const size_t lds = (size_t)2 * prm.R * L.Us * sizeof(double);
-  if (lds > 64 * 1024) return MI_TRANSDUCER_INVALID_VALUE;
+  if (lds > 160 * 1024) return MI_TRANSDUCER_INVALID_VALUE;  // e.g. U = 1024 with a longest duration above 8
 #define LAUNCH_TLAT(KK)                                                                                              \
+  if (lds > 48 * 1024 &&                                                                                             \
+      hipFuncSetAttribute((const void*)tdt_lattice_kernel<KK>, hipFuncAttributeMaxDynamicSharedMemorySize,           \
+                          (int)lds) != hipSuccess)                                                                   \
+    return MI_TRANSDUCER_LAUNCH_FAILURE;                                                                             \
   hipLaunchKernelGGL(tdt_lattice_kernel<KK>, dim3(grid), dim3(64), lds, c.stream, arcs, alphas, betas, ll, costs,    \
                      c.act_lens, c.label_lens, c.T, c.U, L.ND, L.A, cost_scale_of(lambda), with_betas, prm)
   switch (L.K) {
@@ -2853,8 +2944,13 @@ int run_multiblank_lattice(const Common& c, float* costs, float lambda, int with
   const unsigned grid = (unsigned)(with_betas ? 2 * c.B : c.B);
   const int nbc = prm.NB <= 1 ? 1 : (prm.NB <= 2 ? 2 : (prm.NB <= 4 ? 4 : 8));
   const size_t lds = (size_t)prm.R * (2 + nbc) * L.Us * sizeof(double);  // the alpha ring is the larger one
-  if (lds > 160 * 1024) return MI_TRANSDUCER_INVALID_VALUE;
   ProfScope prof(MI_PROFILE_LATTICE, c.stream);
+  if (lds > 160 * 1024) {  // the ring does not fit LDS: pull from global memory instead
+    hipLaunchKernelGGL(multiblank_lattice_pull_kernel, dim3(grid), dim3(L.Us), 0, c.stream, arcs, alphas, betas, ll,
+                       costs, c.act_lens, c.label_lens, c.T, c.U, L.ND, L.Us, L.A, cost_scale_of(lambda), with_betas,
+                       prm);
+    return launch_status();
+  }
 #define LAUNCH_MB_T(NN, TT)                                                                                         \
   do {                                                                                                              \
     if (lds > 48 * 1024 && hipFuncSetAttribute((const void*)multiblank_lattice_kernel<NN, TT>,                      \
@@ -3232,7 +3328,9 @@ int mi_transducer_describe_plan(int act_dtype, int B, int T, int U, int V, int D
   const bool mb = num_big_blanks > 0;
   if (mb) {
     const int nbc = num_big_blanks <= 1 ? 1 : (num_big_blanks <= 2 ? 2 : (num_big_blanks <= 4 ? 4 : 8));
-    snprintf(lattice, sizeof lattice, "multiblank_lattice_kernel<NBC=%d>", nbc);
+    const size_t lds = (size_t)(max_duration + 1) * (2 + nbc) * c.L.Us * sizeof(double);
+    if (lds > 160 * 1024) snprintf(lattice, sizeof lattice, "multiblank_lattice_pull_kernel");
+    else snprintf(lattice, sizeof lattice, "multiblank_lattice_kernel<NBC=%d>", nbc);
   } else if (D == 0 || use_plain_rnnt) {
     snprintf(lattice, sizeof lattice, "rnnt_lattice_kernel<K=%d>", c.L.K);
   } else {

@@ -81,6 +81,19 @@ def test_label_axis_sizes(U):
     check_against_oracle(acts, labels, np.array([T, 5]), np.array([U - 1, (U - 1) // 2]), V - 1, durs, 0.1)
 
 
+@pytest.mark.parametrize("U,durs", [(300, [2, 3, 4, 5, 6, 7, 8, 9]), (513, [2, 4, 8]), (1024, [2, 4]), (1024, [2, 3, 4, 5, 6, 7, 8, 9])])
+def test_label_axes_whose_ring_exceeds_lds(U, durs):
+    """When (longest big blank + 1) x (2 + big blanks) x U doubles pass 160 KB the lattice is computed by the
+    kernel that pulls alphas / betas from global memory; its values are those of the LDS-ring kernel."""
+    rng = np.random.RandomState(U + len(durs))
+    B, T = 2, 23
+    V = 7 + len(durs)
+    acts = rng.randn(B, T, U, V)
+    labels = rng.randint(0, V - 1 - len(durs), size=(B, U - 1))
+    # hundreds of log-sum-exp steps of up to ten terms: float rounding of the gradients reaches 5e-6 (the bar is 1e-4)
+    check_against_oracle(acts, labels, np.array([T, 14]), np.array([U - 1, (U - 1) // 2]), V - 1, durs, 0.05, grad_atol=1e-5)
+
+
 def test_blank_in_the_middle_and_reductions_and_half_precision():
     rng = np.random.RandomState(77)
     B, T, U, V = 3, 10, 5, 12

@@ -71,6 +71,18 @@ def test_label_axis_sizes(U):
     check_against_oracle(acts, labels, [T, 5], [U - 1, (U - 1) // 3], V - 1, durations, 0.02)
 
 
+@pytest.mark.parametrize("U,durations", [(300, [0, 1, 2, 3, 4]), (513, [0, 1, 2, 3, 4, 5, 6, 7, 8]), (1024, [0, 1, 2, 4, 8])])
+def test_label_axes_beyond_the_paired_lattice_kernel(U, durations):
+    """More than 256 label columns run the one-wave-per-direction lattice kernel, whose ring of arc scores
+    grows with U and the longest duration (up to the whole LDS of a CU at U = 1024, durations to 8)."""
+    rng = np.random.RandomState(U)
+    B, T, V = 2, 17, 6
+    acts = rng.randn(B, T, U, V + len(durations))
+    labels = rng.randint(0, V - 1, size=(B, U - 1))
+    # 500+ log-sum-exp steps of up to nine terms each: float rounding of the gradients reaches 2e-6 (the bar is 1e-4)
+    check_against_oracle(acts, labels, [T, 11], [U - 1, (U - 1) // 3], V - 1, durations, 0.02, grad_atol=1e-5)
+
+
 def test_stage_level_lattice():
     # shape of utils/test_gpu_rnnt_kernel.py:617-708: [1,15,11,3] token + [1,15,11,3] duration logits
     rng = np.random.RandomState(0)

@@ -78,6 +78,10 @@ def test_kernel_plan_of_the_documented_shapes(built_lib):
     p = plan(F32, 16, 375, 121, 1028, num_big_blanks=3)  # multi-blank: three big blanks inside V
     assert p["lattice"] == "multiblank_lattice_kernel<NBC=4>" and p["cells"] == "multiblank_cell_kernel"
     assert p["gradient"] == "grad_block_kernel<f32, RT=256, NVT=2, coef> + multiblank_fixup_kernel"
+    p = plan(F32, 2, 50, 1024, 1028, max_duration=8, num_big_blanks=3)  # ring of 9 x 6 x 1024 doubles > 160 KB of LDS
+    assert p["lattice"] == "multiblank_lattice_pull_kernel"
+    p = plan(F32, 2, 50, 513, 1025, D=9, max_duration=8)  # beyond 256 label columns: a wave per direction
+    assert p["lattice"].startswith("tdt_lattice_kernel<K=")
     with pytest.raises(RuntimeError):
         plan(7, 1, 1, 1, 5)
     with pytest.raises(RuntimeError):
