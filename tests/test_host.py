@@ -54,19 +54,19 @@ def test_kernel_plan_of_the_documented_shapes(built_lib):
     plan = _native.describe_plan
     p = plan(F32, 16, 375, 121, 1025)  # the benchmark shape: 256 whole vectors per row
     assert p == {
-        "denominators": "denom_rows_kernel<f32, R=4>",
+        "denominators": "denom_rows_kernel<f32, R=4, RPW=1>",
         "lattice": "rnnt_lattice_kernel<K=2>",
         "cells": "-",
         "gradient": "grad_block_kernel<f32, RT=128, NVT=2, fused>",
     }
     p = plan(BF16, 32, 750, 201, 1025)  # 128 whole vectors of 8 bf16
-    assert p["denominators"] == "denom_rows_kernel<bf16, R=2>" and p["lattice"] == "rnnt_lattice_kernel<K=4>"
+    assert p["denominators"] == "denom_rows_kernel<bf16, R=2, RPW=2>" and p["lattice"] == "rnnt_lattice_kernel<K=4>"
     assert p["gradient"] == "grad_block_kernel<bf16, RT=64, NVT=2, fused>"
     p = plan(F32, 8, 250, 101, 16385)  # 4096 vectors: a workgroup per row
     assert p["denominators"] == "denom_block_kernel<f32, RT=1024, NVT=4>"
     assert p["gradient"] == "grad_block_kernel<f32, RT=1024, NVT=4, fused>"
     p = plan(F32, 4, 50, 21, 29)  # character vocabulary: a wave per row does everything
-    assert p["denominators"] == "denom_rows_kernel<f32, R=1>" and p["gradient"] == "grad_rows_kernel<f32, R=1, fused>"
+    assert p["denominators"] == "denom_rows_kernel<f32, R=1, RPW=4>" and p["gradient"] == "grad_rows_kernel<f32, R=1, fused>"
     p = plan(F32, 2, 10, 5, 40001)  # beyond 8 vectors per thread: the streaming kernels with a running max
     assert p["denominators"] == "denom_gather_kernel<f32>" and p["gradient"] == "grad_stream_kernel<f32>"
     assert p["cells"] == "rnnt_cell_kernel"
