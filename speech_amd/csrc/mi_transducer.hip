@@ -90,7 +90,7 @@ int mi_rnnt_backward(const void* acts, int act_dtype, const int64_t* labels, con
                         workspace_bytes, stream, &c);
   if (st) return st;
   const ScaleArg sc = {grad_scale, grad_scale_stride, grad_mul};
-  const bool fused = grad_rows_R(c, grads) != 0 || grad_block_plan(c, grads).RT != 0;
+  const bool fused = rnnt_rows_fused(c, grads);
   if (!fused && (st = run_rnnt_cells(c, sc, fastemit_lambda, clamp))) return st;
   return run_grad_stream(c, grads, padding_zeroed ? kFlagPaddingDone : 0, fused, sc, fastemit_lambda, clamp);
 }
@@ -140,7 +140,7 @@ int mi_tdt_backward(const void* acts, int act_dtype, const int64_t* labels, cons
   if (st) return st;
   const ScaleArg sc = {grad_scale, grad_scale_stride, grad_mul};
   if (use_plain_rnnt) {  // gpu_rnnt.py:646-682: token gradient from the RNNT kernel, duration gradient stays zero
-    const bool fused = grad_rows_R(c, grads) != 0 || grad_block_plan(c, grads).RT != 0;
+    const bool fused = rnnt_rows_fused(c, grads);
     if (!fused && (st = run_rnnt_cells(c, sc, fastemit_lambda, clamp))) return st;
     return run_grad_stream(c, grads, kFlagZeroDurations | pad_flag, fused, sc, fastemit_lambda, clamp);
   }
@@ -391,7 +391,7 @@ int mi_transducer_describe_plan(int act_dtype, int B, int T, int U, int V, int D
   }
   // a gradient buffer at the 16-byte phase of the logits is assumed (what every allocator returns)
   const BlockPlan gp = grad_block_plan(c, nullptr);
-  const bool fused = !tdt && !mb && (gp.RT != 0 || rows_R(c) != 0);
+  const bool fused = !tdt && !mb && rnnt_rows_fused(c, nullptr);
   snprintf(cells, sizeof cells, "%s", fused ? "-" : (mb ? "multiblank_cell_kernel" : (tdt ? "tdt_cell_kernel" : "rnnt_cell_kernel")));
   if (gp.RT) snprintf(grad, sizeof grad, "grad_block_kernel<%s, RT=%d, NVT=%d, %s>", dt, gp.RT, gp.NVT, fused ? "fused" : "coef");
   else if (rows_R(c)) snprintf(grad, sizeof grad, "grad_rows_kernel<%s, R=%d, %s>", dt, rows_R(c), fused ? "fused" : "coef");

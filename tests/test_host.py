@@ -65,8 +65,9 @@ def test_kernel_plan_of_the_documented_shapes(built_lib):
     p = plan(F32, 8, 250, 101, 16385)  # 4096 vectors: a workgroup per row
     assert p["denominators"] == "denom_block_kernel<f32, RT=1024, NVT=4>"
     assert p["gradient"] == "grad_block_kernel<f32, RT=1024, NVT=4, fused>"
-    p = plan(F32, 4, 50, 21, 29)  # character vocabulary: a wave per row does everything
-    assert p["denominators"] == "denom_rows_kernel<f32, R=1, RPW=4>" and p["gradient"] == "grad_rows_kernel<f32, R=1, fused>"
+    p = plan(F32, 4, 50, 21, 29)  # character vocabulary: short rows, coefficients from the cell kernel
+    assert p["denominators"] == "denom_rows_kernel<f32, R=1, RPW=4>" and p["gradient"] == "grad_rows_kernel<f32, R=1, coef>"
+    assert p["cells"] == "rnnt_cell_kernel"
     p = plan(F32, 2, 10, 5, 40001)  # beyond 8 vectors per thread: the streaming kernels with a running max
     assert p["denominators"] == "denom_gather_kernel<f32>" and p["gradient"] == "grad_stream_kernel<f32>"
     assert p["cells"] == "rnnt_cell_kernel"
