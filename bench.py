@@ -71,23 +71,31 @@ def cpu_baseline(cfg, acts, labels, act_lens, label_lens, n_utt):
     al = act_lens[:n_utt].cpu().numpy()
     ll = label_lens[:n_utt].cpu().numpy()
     lam, clamp = cfg.fastemit_lambda, max(cfg.clamp, 0.0)
-    t0 = time.perf_counter()
-    if cfg.D:
-        oracle.tdt_loss(x, lab, al, ll, cfg.blank, cfg.durations, cfg.sigma, lam, clamp, dtype=np.float32,
-                        num_threads=threads)  # fmt: skip
-    elif cfg.big_blank_durations:
-        oracle.multiblank_loss(x, lab, al, ll, cfg.blank, cfg.big_blank_durations, cfg.sigma, lam, clamp,
-                               dtype=np.float32, num_threads=threads)  # fmt: skip
-    else:
-        oracle.rnnt_cpu_path(x, lab, al, ll, cfg.blank, lam, clamp, dtype=np.float32, num_threads=threads)
+
+    def one_pass():
+        if cfg.D:
+            oracle.tdt_loss(x, lab, al, ll, cfg.blank, cfg.durations, cfg.sigma, lam, clamp, dtype=np.float32,
+                            num_threads=threads)  # fmt: skip
+        elif cfg.big_blank_durations:
+            oracle.multiblank_loss(x, lab, al, ll, cfg.blank, cfg.big_blank_durations, cfg.sigma, lam, clamp,
+                                   dtype=np.float32, num_threads=threads)  # fmt: skip
+        else:
+            oracle.rnnt_cpu_path(x, lab, al, ll, cfg.blank, lam, clamp, dtype=np.float32, num_threads=threads)
+
+    # whole passes until about 20 core-seconds of work are spent (at most 8 passes)
+    passes, t0 = 0, time.perf_counter()
+    while passes < 8 and (passes == 0 or (time.perf_counter() - t0) * threads < 20.0):
+        one_pass()
+        passes += 1
     dt = time.perf_counter() - t0
     return {
-        "value": x.size / dt,
+        "value": passes * x.size / dt,
         "unit": "logit elems/s",
         "cores": threads,
         "kind": "port",
-        "sample": f"first {n_utt} of {cfg.B} utterances of the same batch, full T x U x V, one pass, {dt:.2f} s wall",
-    }
+        "sample": f"first {n_utt} of {cfg.B} utterances of the same batch, full T x U x V, {passes} pass(es), "
+                  f"{dt:.2f} s wall on {threads} threads",
+    }  # fmt: skip
 
 
 def cpu_baseline_logprobs(cfg, acts, labels, act_lens, label_lens, g_target, g_blank, n_utt):
