@@ -180,13 +180,13 @@ JOINT_HIDDEN = 640  # joint_hidden of the reference's FastConformer transducer c
 
 
 def run_joint(args, torch, dev, cfg, labels, act_lens, label_lens):
-    """--op joint: one step = joint_rnnt_loss forward + backward (gradients of f, g, weight, bias)."""
-    import numpy as np
-
+    """--op joint: one step = joint_rnnt_loss (joint_tdt_loss for the TDT workload) forward + backward
+    (gradients of f, g, weight, bias)."""
     from speech_amd import _native
-    from speech_amd.joint import joint_rnnt_loss
+    from speech_amd.joint import joint_rnnt_loss, joint_tdt_loss
 
-    B, T, U, V, H = cfg.B, cfg.T, cfg.U, cfg.V, JOINT_HIDDEN
+    B, T, U, H = cfg.B, cfg.T, cfg.U, JOINT_HIDDEN
+    V = cfg.V + cfg.D  # outputs of the joint's Linear layer (token logits, then duration logits)
     gen = torch.Generator(device=dev).manual_seed(1234)
     f = torch.randn(B, T, H, device=dev, generator=gen).to(torch.bfloat16).requires_grad_(True)
     g = torch.randn(B, U, H, device=dev, generator=gen).to(torch.bfloat16).requires_grad_(True)
@@ -197,15 +197,19 @@ def run_joint(args, torch, dev, cfg, labels, act_lens, label_lens):
     def step():
         for p in (f, g, weight, bias):
             p.grad = None
-        costs = joint_rnnt_loss(f, g, weight, bias, labels, act_lens, label_lens, cfg.blank, cfg.fastemit_lambda,
-                                max(cfg.clamp, 0.0))  # fmt: skip
+        if cfg.D:
+            costs = joint_tdt_loss(f, g, weight, bias, labels, act_lens, label_lens, cfg.blank, cfg.durations, cfg.sigma,
+                                   cfg.fastemit_lambda, max(cfg.clamp, 0.0))  # fmt: skip
+        else:
+            costs = joint_rnnt_loss(f, g, weight, bias, labels, act_lens, label_lens, cfg.blank, cfg.fastemit_lambda,
+                                    max(cfg.clamp, 0.0))  # fmt: skip
         costs.sum().backward()
         return costs
 
     for _ in range(args.warmup):
         step()
     torch.cuda.synchronize()
-    _native.profile_enable(args.steps, ["denominator_pass", "lattice", "gradient_pass"])
+    _native.profile_enable(args.steps, ["denominator_pass", "lattice", "cells", "gradient_pass"])
     t0 = time.perf_counter()
     for _ in range(args.steps):
         costs = step()
@@ -220,7 +224,7 @@ def run_joint(args, torch, dev, cfg, labels, act_lens, label_lens):
     flops = 2.0 * valid * V * H
     achieved = flops / grad_s / 1e12
     result = {
-        "metric": "fused joint + RNNT loss fwd+bwd: logit elems/s and achieved MFMA TFLOP/s vs peak",
+        "metric": "fused joint + %s loss fwd+bwd: logit elems/s and achieved MFMA TFLOP/s vs peak" % ("TDT" if cfg.D else "RNNT"),
         "value": cfg.elems / (ms_per_step * 1e-3),
         "unit": "logit elems/s",
         "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": ms_per_step,
@@ -243,7 +247,8 @@ def run_joint(args, torch, dev, cfg, labels, act_lens, label_lens):
         x = (f[:1, :Tb].detach().float().cpu().numpy(), g[:1, :Ub].detach().float().cpu().numpy(),
              weight.detach().cpu().numpy(), bias.detach().cpu().numpy())  # fmt: skip
         t0 = time.perf_counter()
-        oracle.joint_rnnt_loss(*x, labels[:1, : Ub - 1].cpu().numpy(), [Tb], [Ub - 1], cfg.blank)
+        oracle.joint_rnnt_loss(*x, labels[:1, : Ub - 1].cpu().numpy(), [Tb], [Ub - 1], cfg.blank,
+                               durations=cfg.durations if cfg.D else None, sigma=cfg.sigma)
         dt = time.perf_counter() - t0
         result["cpu_baseline"] = {
             "value": Tb * Ub * V / dt, "unit": "logit elems/s", "cores": 1, "kind": "port",
@@ -273,8 +278,8 @@ def main():
 
     cfg, acts, labels, act_lens, label_lens = synthetic.make_inputs(args.workload, device=dev, generate_on_device=True)
     if args.op == "joint":
-        if cfg.D or cfg.big_blank_durations:
-            print("bench.py: --op joint runs on the RNNT workloads", file=sys.stderr)
+        if cfg.big_blank_durations:
+            print("bench.py: --op joint runs on the RNNT and TDT workloads", file=sys.stderr)
             sys.exit(2)
         del acts
         return run_joint(args, torch, dev, cfg, labels, act_lens, label_lens)

@@ -209,13 +209,22 @@ int mi_rnnt_logprobs_backward(const void* logits, int act_dtype, const int64_t* 
  * Dropout of the hidden activations (the joint network's Dropout(p) between activation and Linear, :1772-1776):
  * dropout_p in [0, 1), 0 = none.  The keep mask is a pure function of (dropout_seed, cell, hidden unit): the
  * backward calls below must be given the same two values and then see the same mask; kept activations are scaled
- * by 1 / (1 - p).  mi_joint_dropout_mask writes that mask ([B*T*U][H] bytes, 1 = kept) for tests. */
-int mi_joint_workspace_bytes(int B, int T, int U, int H, int V, size_t* out_bytes);
+ * by 1 / (1 - p).  mi_joint_dropout_mask writes that mask ([B*T*U][H] bytes, 1 = kept) for tests.
+ * TDT (mi_joint_tdt_*): the Linear layer has V + D outputs, the token logits followed by the D duration logits
+ * (rnnt_pytorch.py:563-568; D <= 8), weight [V+D,H], bias [V+D]; the token softmax covers the first V, the duration
+ * logits are normalised among themselves, and the lattice is the TDT one (durations_host, sigma as mi_tdt_forward).
+ * Every mi_joint_* call on a workspace takes the same D (0 for RNNT): it is part of the workspace layout. */
+int mi_joint_workspace_bytes(int B, int T, int U, int H, int V, int D, size_t* out_bytes);
 int mi_joint_rnnt_forward(const void* f, const void* g, const void* weight, const void* bias, int weight_dtype,
                           const int64_t* labels, const int64_t* act_lens, const int64_t* label_lens, float* costs,
                           int* tile_count, float dropout_p, unsigned long long dropout_seed, int B, int T, int U, int H,
                           int V, int blank, float fastemit_lambda, int with_betas, void* workspace,
                           size_t workspace_bytes, void* stream);
+int mi_joint_tdt_forward(const void* f, const void* g, const void* weight, const void* bias, int weight_dtype,
+                         const int64_t* labels, const int64_t* act_lens, const int64_t* label_lens, float* costs,
+                         int* tile_count, float dropout_p, unsigned long long dropout_seed, int B, int T, int U, int H,
+                         int V, int D, const int32_t* durations_host, int blank, float fastemit_lambda, float sigma,
+                         int with_betas, void* workspace, size_t workspace_bytes, void* stream);
 int mi_joint_dropout_mask(unsigned char* mask, float dropout_p, unsigned long long dropout_seed, int B, int T, int U,
                           int H, void* stream);
 
@@ -229,7 +238,9 @@ int mi_joint_dropout_mask(unsigned char* mask, float dropout_p, unsigned long lo
  *   1, 1 and zeros, so that column H of dlogits^T . hidden is the gradient of the bias.
  * `tiles` is the number of 128-row tiles the two buffers hold: at least what mi_joint_rnnt_forward wrote to
  * tile_count (device int32, nullable there), whose workspace this call needs unchanged (forward with
- * with_betas != 0). */
+ * with_betas != 0).
+ * TDT: dlogits has padded_vocabulary(V + D) columns, columns V .. V+D-1 the gradient of the duration logits
+ * (gpu_rnnt_kernel.py:1244-1439 followed by the log_softmax backward); no clamp on those, as in the reference. */
 int mi_joint_padded_vocabulary(int V);
 int mi_joint_rnnt_backward_logits(const void* f, const void* g, const int64_t* labels, const int64_t* act_lens,
                                   const int64_t* label_lens, void* dlogits, void* hidden, int tiles,
@@ -237,6 +248,12 @@ int mi_joint_rnnt_backward_logits(const void* f, const void* g, const int64_t* l
                                   float grad_mul, float dropout_p, unsigned long long dropout_seed, int B, int T, int U,
                                   int H, int V, int blank, float fastemit_lambda, float clamp, void* workspace,
                                   size_t workspace_bytes, void* stream);
+int mi_joint_tdt_backward_logits(const void* f, const void* g, const int64_t* labels, const int64_t* act_lens,
+                                 const int64_t* label_lens, void* dlogits, void* hidden, int tiles,
+                                 const float* grad_scale, int grad_scale_stride, float grad_mul, float dropout_p,
+                                 unsigned long long dropout_seed, int B, int T, int U, int H, int V, int D,
+                                 const int32_t* durations_host, int blank, float fastemit_lambda, float clamp,
+                                 float sigma, void* workspace, size_t workspace_bytes, void* stream);
 
 /* Backward of the fused joint, last step: d_hidden [rows][H] bf16 (= dlogits . weight, rows as above) times the
  * ReLU derivative, summed over u into d_f [B,T,H] and over t into d_g [B,U,H] (float32; either may be NULL; frames
@@ -245,13 +262,13 @@ int mi_joint_rnnt_backward_logits(const void* f, const void* g, const int64_t* l
  * call's. */
 int mi_joint_reduce_hidden(const void* d_hidden, const void* f, const void* g, const int64_t* act_lens,
                            const int64_t* label_lens, float* d_f, float* d_g, int tiles, float dropout_p,
-                           unsigned long long dropout_seed, int B, int T, int U, int H, int V, void* workspace,
+                           unsigned long long dropout_seed, int B, int T, int U, int H, int V, int D, void* workspace,
                            size_t workspace_bytes, void* stream);
 
 /* Where the forward call left the packed weights inside its workspace: *rows x *pitch bf16, row n = weight[n, :]
- * followed by the bias columns (rows beyond V are zero in the first H columns), so that the d_hidden product can
- * read them in place. */
-int mi_joint_packed_weights(const void* workspace, size_t workspace_bytes, int B, int T, int U, int H, int V,
+ * followed by the bias columns (rows beyond V + D are zero in the first H columns), so that the d_hidden product
+ * can read them in place. */
+int mi_joint_packed_weights(const void* workspace, size_t workspace_bytes, int B, int T, int U, int H, int V, int D,
                             const void** packed, int* rows, int* pitch);
 
 /* Stage-level read-out for kernel parity tests (the reference tests launch each

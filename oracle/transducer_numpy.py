@@ -644,16 +644,18 @@ def bf16_round(x):
 
 
 def joint_rnnt_loss(f, g, weight, bias, labels, act_lens, label_lens, blank, fastemit_lambda=0.0, clamp=0.0, grad_costs=None,
-                    keep_mask=None, dropout_p=0.0):
-    """RNNT loss of the ReLU joint's logits under bf16-autocast arithmetic, and its gradients.
+                    keep_mask=None, dropout_p=0.0, durations=None, sigma=0.0):
+    """RNNT (or, with `durations`, TDT) loss of the ReLU joint's logits under bf16-autocast arithmetic, and its gradients.
 
     logits[b,t,u,:] = drop(relu(bf16(f[b,t] + g[b,u]))) @ bf16(weight).T + bias   (modules/rnnt.py:1707-1724,
     joint_net = ReLU, Dropout, Linear :1766-1777; operands rounded to bf16, products and sums exact here --
     float32 accumulation on the GPU; the bias enters as bf16(bias) + bf16(bias - bf16(bias)), i.e. to about
     16 bits).  drop(x) = bf16(x * keep_mask / (1 - dropout_p)) for a given boolean keep_mask [B,T,U,H]
     (torch.nn.functional.dropout's definition; which units are kept is the caller's business), identity without
-    one.  The loss and the gradient of the logits are rnnt_loss's; the gradients of f, g, weight, bias follow by the
-    chain rule with every rounding treated as the identity (what autograd does under autocast).
+    one.  The loss and the gradient of the logits are rnnt_loss's -- tdt_loss's when `durations` is given: the
+    Linear layer then has V + len(durations) outputs, token logits first (rnnt_pytorch.py:563-568); the gradients
+    of f, g, weight, bias follow by the chain rule with every rounding treated as the identity (what autograd does
+    under autocast).
     Returns (costs, d_f, d_g, d_weight, d_bias).
     """
     f = bf16_round(f)
@@ -675,7 +677,10 @@ def joint_rnnt_loss(f, g, weight, bias, labels, act_lens, label_lens, blank, fas
         hidden = np.where(keep, bf16_round(hidden.astype(np.float32) * scale), 0.0)
         chain = chain * keep * np.float64(scale)
     logits = hidden @ w.T + b_eff
-    costs, d_logits, _ = rnnt_loss(logits, labels, act_lens, label_lens, blank, fastemit_lambda, clamp)
+    if durations:
+        costs, d_logits, _ = tdt_loss(logits, labels, act_lens, label_lens, blank, durations, sigma, fastemit_lambda, clamp)
+    else:
+        costs, d_logits, _ = rnnt_loss(logits, labels, act_lens, label_lens, blank, fastemit_lambda, clamp)
     if grad_costs is not None:
         d_logits = d_logits * np.asarray(grad_costs, dtype=np.float64).reshape(B, 1, 1, 1)
     d_weight = np.einsum('btuv,btuh->vh', d_logits, hidden)

@@ -1,5 +1,13 @@
 """Joint projection fused into the transducer loss (the [B,T,U,V] tensor is never written)."""
 
-from speech_amd.joint.fused import JointRNNTLoss, joint_dropout_mask, joint_rnnt_forward, joint_rnnt_loss
+from speech_amd.joint.fused import (
+    JointRNNTLoss,
+    joint_dropout_mask,
+    joint_rnnt_forward,
+    joint_rnnt_loss,
+    joint_tdt_forward,
+    joint_tdt_loss,
+)
 
-__all__ = ["JointRNNTLoss", "joint_dropout_mask", "joint_rnnt_forward", "joint_rnnt_loss"]
+__all__ = ["JointRNNTLoss", "joint_dropout_mask", "joint_rnnt_forward", "joint_rnnt_loss", "joint_tdt_forward",
+           "joint_tdt_loss"]  # fmt: skip

@@ -84,3 +84,32 @@ def test_dropout_against_torch_autograd():
                                   keep_mask=np.ones((B, T, U, H), dtype=bool), dropout_p=0.0)  # fmt: skip
     for a, b in zip(plain, ones):
         np.testing.assert_array_equal(a, b)
+
+
+@pytest.mark.parametrize("durations", [[0, 1, 2], [1, 2], [0, 1, 2, 3, 4]])
+def test_tdt_variant_against_torch_autograd(durations):
+    """With `durations` the Linear layer has V + D outputs and the loss is the TDT one: checked against torch autograd
+    of relu / Linear fed with the logits-gradient of an independent alpha-only TDT recursion (helpers.tdt_autograd).
+    f + g is exact in bf16 here (multiples of 1/8 below 4), so no rounding enters."""
+    from helpers import tdt_autograd
+
+    B, T, U, H, V, D, sigma = 2, 4, 3, 16, 6, len(durations), 0.05
+    rng = np.random.RandomState(D)
+    f, g = rng.randint(-16, 17, size=(B, T, H)) / 8.0, rng.randint(-16, 17, size=(B, U, H)) / 8.0
+    w, bias = bf16_round(rng.randn(V + D, H) / 4), bf16_round(rng.randn(V + D))
+    labels = rng.randint(0, V - 1, size=(B, U - 1))
+    gc = rng.rand(B) + 0.5
+    costs, d_f, d_g, d_w, d_b = oracle.joint_rnnt_loss(
+        f, g, w, bias, labels, [T] * B, [U - 1] * B, V - 1, grad_costs=gc, durations=durations, sigma=sigma
+    )
+    ft, gt = torch.tensor(f, requires_grad=True), torch.tensor(g, requires_grad=True)
+    wt, bt = torch.tensor(w, requires_grad=True), torch.tensor(bias, requires_grad=True)
+    logits = torch.nn.functional.linear(torch.relu(ft[:, :, None, :] + gt[:, None, :, :]), wt, bt)
+    d_logits = []
+    for b in range(B):
+        nll, gl = tdt_autograd(logits[b].detach().numpy(), labels[b], V - 1, durations, sigma)
+        np.testing.assert_allclose(costs[b], nll, rtol=1e-10)
+        d_logits.append(gl * gc[b])
+    logits.backward(torch.tensor(np.stack(d_logits)))
+    for got, want in zip((d_f, d_g, d_w, d_b), (ft.grad, gt.grad, wt.grad, bt.grad)):
+        np.testing.assert_allclose(got, want.numpy(), rtol=1e-9, atol=1e-11)
