@@ -144,3 +144,42 @@ def test_rejects_bad_duration_arguments():
         joint_tdt_forward(*args, 3, list(range(9)))  # more than 8 durations
     with pytest.raises(RuntimeError):
         joint_tdt_forward(*args, 9, [0, 2, 3])  # no duration 1 among the first two (gpu_rnnt_kernel.py:1137-1148)
+
+
+@pytest.mark.parametrize("tdt", [False, True])
+def test_backward_agrees_with_autograd_of_the_unfused_pipeline(tdt):
+    """Several tiles per utterance AND nine row blocks of vocabulary (too large for the per-cell oracle loops): the
+    reference's pipeline in float32 on the same GPU -- joint tensor from the bf16-rounded operands, loss module,
+    torch autograd -- against the fused op, gradients at the bf16 tolerance of the other tests."""
+    durations = [0, 1, 2, 3, 4] if tdt else []
+    V, H, B, T, U = 1025, 640, 3, 40, 15
+    f, g, W, bias, labels, al, ll = make_case(11, B, T, U, H, V, len(durations))
+    lab, ald, lld = dev_ints(labels, al, ll)
+    gc = torch.tensor([0.5, 1.0, 1.5], device=DEV)
+
+    def leaves():
+        return (f.to(DEV).requires_grad_(True), g.to(DEV).requires_grad_(True),
+                W.to(torch.bfloat16).float().to(DEV).requires_grad_(True), bias.to(DEV).requires_grad_(True))  # fmt: skip
+
+    fd, gd, Wd, bd = leaves()
+    if tdt:
+        costs = joint_tdt_loss(fd, gd, Wd, bd, lab, ald, lld, V - 1, durations, 0.05, 0.01)
+    else:
+        costs = joint_rnnt_loss(fd, gd, Wd, bd, lab, ald, lld, V - 1, 0.01)
+    (costs * gc).sum().backward()
+    fr, gr, Wr, br = leaves()
+    hidden = torch.relu(fr.unsqueeze(2) + gr.unsqueeze(1)).float()
+    logits = hidden @ Wr.t() + br
+    if tdt:
+        module = TDTLossNumba(blank=V - 1, durations=durations, reduction='none', sigma=0.05, fastemit_lambda=0.01)
+    else:
+        from speech_amd import RNNTLossNumba
+
+        module = RNNTLossNumba(blank=V - 1, reduction='none', fastemit_lambda=0.01)
+    ref = module(logits, lab, ald, lld).float()
+    (ref * gc).sum().backward()
+    np.testing.assert_allclose(costs.detach().cpu().numpy(), ref.detach().cpu().numpy(), rtol=2e-5)
+    for name, x, want in (("d_f", fd.grad, fr.grad), ("d_g", gd.grad, gr.grad), ("d_weight", Wd.grad, Wr.grad),
+                          ("d_bias", bd.grad, br.grad)):  # fmt: skip
+        err = (x.float() - want.float()).abs().max().item()
+        assert err <= 2.0**-6 * want.float().abs().max().item() + 1e-7, (name, err)
