@@ -183,3 +183,30 @@ def test_backward_agrees_with_autograd_of_the_unfused_pipeline(tdt):
                           ("d_bias", bd.grad, br.grad)):  # fmt: skip
         err = (x.float() - want.float()).abs().max().item()
         assert err <= 2.0**-6 * want.float().abs().max().item() + 1e-7, (name, err)
+
+
+@pytest.mark.parametrize("tdt", [False, True])
+def test_fused_sub_batches_give_the_same_costs_and_gradients(tdt):
+    """fused_batch_size (the reference's sub-batch loop, modules/rnnt.py:1527-1587): utterances do not interact, so the
+    costs are the same numbers and the gradients differ by the order of a few bf16-rounded partial sums at most."""
+    durations = [0, 1, 2] if tdt else []
+    V, H, B, T, U = 50, 320, 7, 12, 6
+    f, g, W, bias, labels, al, ll = make_case(12, B, T, U, H, V, len(durations))
+    lab, ald, lld = dev_ints(labels, al, ll)
+
+    def run(fbs):
+        fd, gd = f.to(DEV).requires_grad_(True), g.to(DEV).requires_grad_(True)
+        Wd, bd = W.to(DEV).requires_grad_(True), bias.to(DEV).requires_grad_(True)
+        if tdt:
+            costs = joint_tdt_loss(fd, gd, Wd, bd, lab, ald, lld, V - 1, durations, 0.05, fused_batch_size=fbs)
+        else:
+            costs = joint_rnnt_loss(fd, gd, Wd, bd, lab, ald, lld, V - 1, fused_batch_size=fbs)
+        costs.sum().backward()
+        return costs.detach(), fd.grad.float(), gd.grad.float(), Wd.grad, bd.grad
+
+    whole, parts = run(None), run(3)
+    assert parts[0].shape == (B,) and torch.equal(whole[0], parts[0])
+    for x, y in zip(whole[1:], parts[1:]):
+        assert (x - y).abs().max().item() <= 2.0**-7 * x.abs().max().item()
+    with pytest.raises(ValueError):
+        run(-1)
