@@ -25,6 +25,7 @@
 #include <stdio.h>
 #include <stdint.h>
 
+#include <type_traits>
 #include <vector>
 
 #include "mi_transducer.h"
