@@ -1,0 +1,109 @@
+"""Entry points of the C ABI that the module path does not go through: the stage-by-stage calls (denominators,
+lattice), the TDT function-level seam (tdt_loss_gpu, rnnt.py:239-363), the per-kernel timing hooks and the copy
+probe of the benchmark."""
+
+import numpy as np
+import pytest
+import torch
+
+import oracle
+from speech_amd import _native
+from speech_amd.rnnt_loss import rnnt
+
+from gpu_utils import DEV, to_dev
+
+pytestmark = pytest.mark.gpu
+
+
+def make(seed, B, T, U, V):
+    rng = np.random.RandomState(seed)
+    x = rng.randn(B, T, U, V).astype(np.float32)
+    labels = rng.randint(0, 5, size=(B, U - 1))
+    al, ll = rng.randint(1, T + 1, size=B), rng.randint(0, U, size=B)
+    al[0], ll[-1] = T, U - 1
+    return x, labels, al, ll
+
+
+@pytest.mark.parametrize("with_betas", [False, True])
+def test_denominators_then_lattice_is_the_forward_call(with_betas):
+    B, T, U, V = 3, 13, 8, 70
+    x, labels, al, ll = make(1, B, T, U, V)
+    acts = torch.tensor(x, device=DEV)
+    lab, ald, lld = to_dev(labels, al, ll)
+    whole, split = (torch.empty(B, dtype=torch.float32, device=DEV) for _ in range(2))
+    ws1, ws2 = rnnt.new_workspace(acts), rnnt.new_workspace(acts)
+    rnnt.rnnt_forward(acts, lab, ald, lld, whole, V - 1, 0.01, with_betas, ws1)
+    rnnt.denominators(acts, lab, ald, lld, V - 1, ws2)
+    rnnt.rnnt_lattice(ald, lld, split, B, T, U, 0.01, with_betas, ws2)
+    assert torch.equal(whole, split)
+    c_ref, _, _ = oracle.rnnt_loss(x, labels, al, ll, V - 1, 0.01, 0.0)
+    np.testing.assert_allclose(split.cpu().numpy(), c_ref, rtol=1e-6)
+    # TDT: the same two stages with duration planes
+    durations = [0, 1, 2]
+    rnnt_x = np.random.RandomState(2).randn(B, T, U, V + 3).astype(np.float32)
+    acts = torch.tensor(rnnt_x, device=DEV)
+    ws1, ws2 = rnnt.new_workspace(acts, 3), rnnt.new_workspace(acts, 3)
+    rnnt.tdt_forward(acts, lab, ald, lld, whole, V - 1, durations, 0.0, 0.05, False, with_betas, ws1)
+    rnnt.denominators(acts, lab, ald, lld, V - 1, ws2, 3)
+    rnnt.tdt_lattice(ald, lld, split, B, T, U, durations, 0.0, 0.05, with_betas, ws2)
+    assert torch.equal(whole, split)
+    c_ref, _, _ = oracle.tdt_loss(rnnt_x, labels, al, ll, V - 1, durations, 0.05)
+    np.testing.assert_allclose(split.cpu().numpy(), c_ref, rtol=1e-6)
+
+
+def test_tdt_function_level_seam():
+    B, T, U, V, durations = 3, 9, 5, 12, [0, 1, 2, 3]
+    x, labels, al, ll = make(3, B, T, U, V + len(durations))
+    acts = torch.tensor(x, device=DEV)
+    lab, ald, lld = to_dev(labels, al, ll)
+    costs = torch.zeros(B, device=DEV)
+    grads = torch.full_like(acts, float('nan'))
+    assert rnnt.tdt_loss_gpu(acts, lab, ald, lld, costs, grads, V - 1, durations, 0.01, 0.2, 0, 0.05) is True
+    c_ref, g_ref, _ = oracle.tdt_loss(x, labels, al, ll, V - 1, durations, 0.05, 0.01, 0.2)
+    np.testing.assert_allclose(costs.cpu().numpy(), c_ref, rtol=1e-6)
+    assert np.abs(grads.cpu().numpy() - g_ref).max() < 2e-6
+    # grads None: forward only (rnnt.py:336-345)
+    only = torch.zeros(B, device=DEV)
+    assert rnnt.tdt_loss_gpu(acts, lab, ald, lld, only, None, V - 1, durations, 0.01, 0.2, 0, 0.05) is True
+    assert torch.equal(only, costs)
+    with pytest.raises(TypeError):
+        rnnt.tdt_loss_gpu(acts, lab, ald, lld, costs.double(), None, V - 1, durations, 0.0, 0.0, 0, 0.0)
+
+
+def test_timing_hooks_count_the_launches_they_bracket():
+    B, T, U, V = 2, 7, 4, 33
+    x, labels, al, ll = make(4, B, T, U, V)
+    acts = torch.tensor(x, device=DEV)
+    lab, ald, lld = to_dev(labels, al, ll)
+    costs = torch.empty(B, dtype=torch.float32, device=DEV)
+    grads = torch.empty_like(acts)
+    ws = rnnt.new_workspace(acts)
+    _native.profile_enable(8, ["denominator_pass", "lattice", "gradient_pass"])
+    try:
+        for _ in range(3):
+            rnnt.rnnt_forward(acts, lab, ald, lld, costs, V - 1, 0.0, True, ws)
+            rnnt.rnnt_backward(acts, lab, ald, lld, grads, None, V - 1, 0.0, 0.0, ws)
+        torch.cuda.synchronize()
+        got = _native.profile_read()
+    finally:
+        _native.profile_disable()
+    for name in ("denominator_pass", "lattice", "gradient_pass"):
+        ms, n = got[name]
+        assert n == 3 and 0.0 < ms < 1000.0, (name, ms, n)
+    assert got["zero_padding"][1] == 0
+    # disabled again: nothing is recorded
+    rnnt.rnnt_forward(acts, lab, ald, lld, costs, V - 1, 0.0, True, ws)
+    torch.cuda.synchronize()
+    assert all(n == 0 for _, n in _native.profile_read().values())
+
+
+def test_copy_probe_copies():
+    n = 1 << 20
+    src = torch.randint(0, 255, (n,), dtype=torch.uint8, device=DEV)
+    dst = torch.zeros_like(src)
+    stream = torch.cuda.current_stream().cuda_stream
+    assert _native.lib().mi_transducer_copy_probe(src.data_ptr(), dst.data_ptr(), n, stream) == _native.SUCCESS
+    torch.cuda.synchronize()
+    assert torch.equal(src, dst)
+    assert _native.lib().mi_transducer_copy_probe(src.data_ptr(), dst.data_ptr(), n - 8, stream) == _native.INVALID_VALUE
+    assert _native.lib().mi_transducer_copy_probe(src.data_ptr() + 4, dst.data_ptr(), n - 16, stream) == _native.INVALID_VALUE
