@@ -107,3 +107,30 @@ def test_copy_probe_copies():
     assert torch.equal(src, dst)
     assert _native.lib().mi_transducer_copy_probe(src.data_ptr(), dst.data_ptr(), n - 8, stream) == _native.INVALID_VALUE
     assert _native.lib().mi_transducer_copy_probe(src.data_ptr() + 4, dst.data_ptr(), n - 16, stream) == _native.INVALID_VALUE
+
+
+def test_work_is_enqueued_on_the_current_stream():
+    """The reference picks torch's current stream (rnnt.py:173-176).  Here: inputs produced on a side stream, the
+    loss called there without any synchronisation in between, the result consumed there -- right only if every
+    kernel of forward and backward went to that stream (a slow kernel ahead of the producer makes a miss show)."""
+    from speech_amd import RNNTLossNumba
+
+    B, T, U, V = 4, 40, 12, 257
+    x, labels, al, ll = make(5, B, T, U, V)
+    lab, ald, lld = to_dev(labels, al, ll)
+    base = torch.tensor(x, device=DEV)
+    ref_acts = (base * 2 + 1).requires_grad_(True)
+    ref = RNNTLossNumba(blank=V - 1, reduction='none')(ref_acts, lab, ald, lld)
+    ref.sum().backward()
+    torch.cuda.synchronize()
+    side = torch.cuda.Stream()
+    big = torch.randn(4096, 4096, device=DEV)
+    with torch.cuda.stream(side):
+        for _ in range(20):
+            big = big @ big * 1e-3  # keeps the side stream busy ahead of the producer below
+        acts = (base * 2 + 1).requires_grad_(True)
+        costs = RNNTLossNumba(blank=V - 1, reduction='none')(acts, lab, ald, lld)
+        costs.sum().backward()
+        got_c, got_g = costs.detach().clone(), acts.grad.clone()
+    side.synchronize()
+    assert torch.equal(got_c, ref.detach()) and torch.equal(got_g, ref_acts.grad)
