@@ -183,7 +183,7 @@ def run_joint(args, torch, dev, cfg, labels, act_lens, label_lens):
     """--op joint: one step = joint_rnnt_loss (joint_tdt_loss for the TDT workload) forward + backward
     (gradients of f, g, weight, bias)."""
     from speech_amd import _native
-    from speech_amd.joint import joint_rnnt_loss, joint_tdt_loss
+    from speech_amd.joint import joint_multiblank_loss, joint_rnnt_loss, joint_tdt_loss
 
     B, T, U, H = cfg.B, cfg.T, cfg.U, JOINT_HIDDEN
     V = cfg.V + cfg.D  # outputs of the joint's Linear layer (token logits, then duration logits)
@@ -200,6 +200,9 @@ def run_joint(args, torch, dev, cfg, labels, act_lens, label_lens):
         if cfg.D:
             costs = joint_tdt_loss(f, g, weight, bias, labels, act_lens, label_lens, cfg.blank, cfg.durations, cfg.sigma,
                                    cfg.fastemit_lambda, max(cfg.clamp, 0.0))  # fmt: skip
+        elif cfg.big_blank_durations:
+            costs = joint_multiblank_loss(f, g, weight, bias, labels, act_lens, label_lens, cfg.blank,
+                                          cfg.big_blank_durations, cfg.sigma, cfg.fastemit_lambda, max(cfg.clamp, 0.0))  # fmt: skip
         else:
             costs = joint_rnnt_loss(f, g, weight, bias, labels, act_lens, label_lens, cfg.blank, cfg.fastemit_lambda,
                                     max(cfg.clamp, 0.0))  # fmt: skip
@@ -224,7 +227,7 @@ def run_joint(args, torch, dev, cfg, labels, act_lens, label_lens):
     flops = 2.0 * valid * V * H
     achieved = flops / grad_s / 1e12
     result = {
-        "metric": "fused joint + %s loss fwd+bwd: logit elems/s and achieved MFMA TFLOP/s vs peak" % ("TDT" if cfg.D else "RNNT"),
+        "metric": "fused joint + %s loss fwd+bwd: logit elems/s and achieved MFMA TFLOP/s vs peak" % ("TDT" if cfg.D else ("multi-blank" if cfg.big_blank_durations else "RNNT")),
         "value": cfg.elems / (ms_per_step * 1e-3),
         "unit": "logit elems/s",
         "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": ms_per_step,
@@ -248,7 +251,8 @@ def run_joint(args, torch, dev, cfg, labels, act_lens, label_lens):
              weight.detach().cpu().numpy(), bias.detach().cpu().numpy())  # fmt: skip
         t0 = time.perf_counter()
         oracle.joint_rnnt_loss(*x, labels[:1, : Ub - 1].cpu().numpy(), [Tb], [Ub - 1], cfg.blank,
-                               durations=cfg.durations if cfg.D else None, sigma=cfg.sigma)
+                               durations=cfg.durations if cfg.D else None, sigma=cfg.sigma,
+                               big_blank_durations=cfg.big_blank_durations or None)
         dt = time.perf_counter() - t0
         result["cpu_baseline"] = {
             "value": Tb * Ub * V / dt, "unit": "logit elems/s", "cores": 1, "kind": "port",
@@ -278,9 +282,6 @@ def main():
 
     cfg, acts, labels, act_lens, label_lens = synthetic.make_inputs(args.workload, device=dev, generate_on_device=True)
     if args.op == "joint":
-        if cfg.big_blank_durations:
-            print("bench.py: --op joint runs on the RNNT and TDT workloads", file=sys.stderr)
-            sys.exit(2)
         del acts
         return run_joint(args, torch, dev, cfg, labels, act_lens, label_lens)
     acts.requires_grad_(True)

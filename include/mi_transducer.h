@@ -213,8 +213,11 @@ int mi_rnnt_logprobs_backward(const void* logits, int act_dtype, const int64_t* 
  * TDT (mi_joint_tdt_*): the Linear layer has V + D outputs, the token logits followed by the D duration logits
  * (rnnt_pytorch.py:563-568; D <= 8), weight [V+D,H], bias [V+D]; the token softmax covers the first V, the duration
  * logits are normalised among themselves, and the lattice is the TDT one (durations_host, sigma as mi_tdt_forward).
- * Every mi_joint_* call on a workspace takes the same D (0 for RNNT): it is part of the workspace layout. */
-int mi_joint_workspace_bytes(int B, int T, int U, int H, int V, int D, size_t* out_bytes);
+ * Multi-blank (mi_joint_multiblank_*): V counts the num_big_blanks <= 8 big blanks, which sit at rows blank-1-i of
+ * the one softmax (as in mi_multiblank_forward); the lattice is the multi-blank one.
+ * Every mi_joint_* call on a workspace takes the same D and num_big_blanks (both 0 for RNNT, at most one of them
+ * non-zero): they are part of the workspace layout. */
+int mi_joint_workspace_bytes(int B, int T, int U, int H, int V, int D, int num_big_blanks, size_t* out_bytes);
 int mi_joint_rnnt_forward(const void* f, const void* g, const void* weight, const void* bias, int weight_dtype,
                           const int64_t* labels, const int64_t* act_lens, const int64_t* label_lens, float* costs,
                           int* tile_count, float dropout_p, unsigned long long dropout_seed, int B, int T, int U, int H,
@@ -225,6 +228,12 @@ int mi_joint_tdt_forward(const void* f, const void* g, const void* weight, const
                          int* tile_count, float dropout_p, unsigned long long dropout_seed, int B, int T, int U, int H,
                          int V, int D, const int32_t* durations_host, int blank, float fastemit_lambda, float sigma,
                          int with_betas, void* workspace, size_t workspace_bytes, void* stream);
+int mi_joint_multiblank_forward(const void* f, const void* g, const void* weight, const void* bias, int weight_dtype,
+                                const int64_t* labels, const int64_t* act_lens, const int64_t* label_lens, float* costs,
+                                int* tile_count, float dropout_p, unsigned long long dropout_seed, int B, int T, int U,
+                                int H, int V, int num_big_blanks, const int32_t* big_blank_durations_host, int blank,
+                                float fastemit_lambda, float sigma, int with_betas, void* workspace,
+                                size_t workspace_bytes, void* stream);
 int mi_joint_dropout_mask(unsigned char* mask, float dropout_p, unsigned long long dropout_seed, int B, int T, int U,
                           int H, void* stream);
 
@@ -254,6 +263,13 @@ int mi_joint_tdt_backward_logits(const void* f, const void* g, const int64_t* la
                                  unsigned long long dropout_seed, int B, int T, int U, int H, int V, int D,
                                  const int32_t* durations_host, int blank, float fastemit_lambda, float clamp,
                                  float sigma, void* workspace, size_t workspace_bytes, void* stream);
+int mi_joint_multiblank_backward_logits(const void* f, const void* g, const int64_t* labels, const int64_t* act_lens,
+                                        const int64_t* label_lens, void* dlogits, void* hidden, int tiles,
+                                        const float* grad_scale, int grad_scale_stride, float grad_mul,
+                                        float dropout_p, unsigned long long dropout_seed, int B, int T, int U, int H,
+                                        int V, int num_big_blanks, const int32_t* big_blank_durations_host, int blank,
+                                        float fastemit_lambda, float clamp, float sigma, void* workspace,
+                                        size_t workspace_bytes, void* stream);
 
 /* Backward of the fused joint, last step: d_hidden [rows][H] bf16 (= dlogits . weight, rows as above) times the
  * ReLU derivative, summed over u into d_f [B,T,H] and over t into d_g [B,U,H] (float32; either may be NULL; frames
@@ -262,14 +278,14 @@ int mi_joint_tdt_backward_logits(const void* f, const void* g, const int64_t* la
  * call's. */
 int mi_joint_reduce_hidden(const void* d_hidden, const void* f, const void* g, const int64_t* act_lens,
                            const int64_t* label_lens, float* d_f, float* d_g, int tiles, float dropout_p,
-                           unsigned long long dropout_seed, int B, int T, int U, int H, int V, int D, void* workspace,
-                           size_t workspace_bytes, void* stream);
+                           unsigned long long dropout_seed, int B, int T, int U, int H, int V, int D,
+                           int num_big_blanks, void* workspace, size_t workspace_bytes, void* stream);
 
 /* Where the forward call left the packed weights inside its workspace: *rows x *pitch bf16, row n = weight[n, :]
  * followed by the bias columns (rows beyond V + D are zero in the first H columns), so that the d_hidden product
  * can read them in place. */
 int mi_joint_packed_weights(const void* workspace, size_t workspace_bytes, int B, int T, int U, int H, int V, int D,
-                            const void** packed, int* rows, int* pitch);
+                            int num_big_blanks, const void** packed, int* rows, int* pitch);
 
 /* Stage-level read-out for kernel parity tests (the reference tests launch each
  * kernel on its own, tests/collections/asr/numba/rnnt_loss/utils/test_gpu_rnnt_kernel.py):

@@ -644,8 +644,9 @@ def bf16_round(x):
 
 
 def joint_rnnt_loss(f, g, weight, bias, labels, act_lens, label_lens, blank, fastemit_lambda=0.0, clamp=0.0, grad_costs=None,
-                    keep_mask=None, dropout_p=0.0, durations=None, sigma=0.0):
-    """RNNT (or, with `durations`, TDT) loss of the ReLU joint's logits under bf16-autocast arithmetic, and its gradients.
+                    keep_mask=None, dropout_p=0.0, durations=None, sigma=0.0, big_blank_durations=None):
+    """RNNT (with `durations` TDT, with `big_blank_durations` multi-blank) loss of the ReLU joint's logits under
+    bf16-autocast arithmetic, and its gradients.
 
     logits[b,t,u,:] = drop(relu(bf16(f[b,t] + g[b,u]))) @ bf16(weight).T + bias   (modules/rnnt.py:1707-1724,
     joint_net = ReLU, Dropout, Linear :1766-1777; operands rounded to bf16, products and sums exact here --
@@ -679,6 +680,9 @@ def joint_rnnt_loss(f, g, weight, bias, labels, act_lens, label_lens, blank, fas
     logits = hidden @ w.T + b_eff
     if durations:
         costs, d_logits, _ = tdt_loss(logits, labels, act_lens, label_lens, blank, durations, sigma, fastemit_lambda, clamp)
+    elif big_blank_durations:
+        costs, d_logits, _ = multiblank_loss(logits, labels, act_lens, label_lens, blank, big_blank_durations, sigma,
+                                             fastemit_lambda, clamp)
     else:
         costs, d_logits, _ = rnnt_loss(logits, labels, act_lens, label_lens, blank, fastemit_lambda, clamp)
     if grad_costs is not None:

@@ -16,7 +16,7 @@ INCLUDE_DIR = os.path.join(os.path.dirname(_HERE), "include")
 LIB_PATH = os.environ.get("MI_TRANSDUCER_LIB") or os.path.join(CSRC_DIR, "libmi_transducer.so")
 SOURCES = [os.path.join(CSRC_DIR, "mi_transducer.hip")]
 
-ABI_VERSION = 12
+ABI_VERSION = 13
 SUCCESS, INVALID_VALUE, LAUNCH_FAILURE = 0, 1, 2
 DTYPE_F32, DTYPE_BF16, DTYPE_F16 = 0, 1, 2
 
@@ -77,12 +77,15 @@ _SIGNATURES = {
                                  _c_size_t, _vp],
     "mi_rnnt_logprobs_backward": [_vp, _c_int, _vp, _vp, _vp, _vp, _vp, _vp, _c_int, _c_int, _c_int, _c_int, _c_int,
                                   _c_int, _vp, _c_size_t, _vp],
-    "mi_joint_workspace_bytes": [_c_int, _c_int, _c_int, _c_int, _c_int, _c_int, ctypes.POINTER(_c_size_t)],
+    "mi_joint_workspace_bytes": [_c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, ctypes.POINTER(_c_size_t)],
     "mi_joint_rnnt_forward": [_vp, _vp, _vp, _vp, _c_int, _vp, _vp, _vp, _vp, _vp, _c_float, ctypes.c_uint64, _c_int,
                               _c_int, _c_int, _c_int, _c_int, _c_int, _c_float, _c_int, _vp, _c_size_t, _vp],
     "mi_joint_tdt_forward": [_vp, _vp, _vp, _vp, _c_int, _vp, _vp, _vp, _vp, _vp, _c_float, ctypes.c_uint64, _c_int,
                              _c_int, _c_int, _c_int, _c_int, _c_int, _vp, _c_int, _c_float, _c_float, _c_int, _vp,
                              _c_size_t, _vp],
+    "mi_joint_multiblank_forward": [_vp, _vp, _vp, _vp, _c_int, _vp, _vp, _vp, _vp, _vp, _c_float, ctypes.c_uint64,
+                                    _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _vp, _c_int, _c_float, _c_float,
+                                    _c_int, _vp, _c_size_t, _vp],
     "mi_joint_dropout_mask": [_vp, _c_float, ctypes.c_uint64, _c_int, _c_int, _c_int, _c_int, _vp],
     "mi_joint_padded_vocabulary": [_c_int],
     "mi_joint_rnnt_backward_logits": [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _c_int, _vp, _c_int, _c_float,
@@ -91,9 +94,13 @@ _SIGNATURES = {
     "mi_joint_tdt_backward_logits": [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _c_int, _vp, _c_int, _c_float,
                                      _c_float, ctypes.c_uint64, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _vp,
                                      _c_int, _c_float, _c_float, _c_float, _vp, _c_size_t, _vp],
+    "mi_joint_multiblank_backward_logits": [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _c_int, _vp, _c_int, _c_float,
+                                            _c_float, ctypes.c_uint64, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int,
+                                            _vp, _c_int, _c_float, _c_float, _c_float, _vp, _c_size_t, _vp],
     "mi_joint_reduce_hidden": [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _c_int, _c_float, ctypes.c_uint64, _c_int, _c_int,
-                               _c_int, _c_int, _c_int, _c_int, _vp, _c_size_t, _vp],
-    "mi_joint_packed_weights": [_vp, _c_size_t, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, ctypes.POINTER(_vp),
+                               _c_int, _c_int, _c_int, _c_int, _c_int, _vp, _c_size_t, _vp],
+    "mi_joint_packed_weights": [_vp, _c_size_t, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int,
+                                ctypes.POINTER(_vp),
                                 ctypes.POINTER(_c_int), ctypes.POINTER(_c_int)],
     "mi_transducer_export_lattice": [_vp, _c_size_t, _vp, _vp, _c_int, _c_int, _c_int, _c_int, _vp, _vp, _vp, _vp,
                                      _vp, _vp],

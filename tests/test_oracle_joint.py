@@ -113,3 +113,32 @@ def test_tdt_variant_against_torch_autograd(durations):
     logits.backward(torch.tensor(np.stack(d_logits)))
     for got, want in zip((d_f, d_g, d_w, d_b), (ft.grad, gt.grad, wt.grad, bt.grad)):
         np.testing.assert_allclose(got, want.numpy(), rtol=1e-9, atol=1e-11)
+
+
+@pytest.mark.parametrize("big_blanks", [[2], [2, 4], [2, 3, 5]])
+def test_multiblank_variant_against_torch_autograd(big_blanks):
+    """With `big_blank_durations` the loss is the multi-blank one (big blanks at outputs blank-1-i of the same
+    softmax): checked as the TDT variant above, with helpers.multiblank_autograd as the independent recursion."""
+    from helpers import multiblank_autograd
+
+    B, T, U, H, sigma = 2, 5, 3, 16, 0.05
+    V = 5 + len(big_blanks) + 1
+    rng = np.random.RandomState(len(big_blanks))
+    f, g = rng.randint(-16, 17, size=(B, T, H)) / 8.0, rng.randint(-16, 17, size=(B, U, H)) / 8.0
+    w, bias = bf16_round(rng.randn(V, H) / 4), bf16_round(rng.randn(V))
+    labels = rng.randint(0, 5, size=(B, U - 1))
+    gc = rng.rand(B) + 0.5
+    costs, d_f, d_g, d_w, d_b = oracle.joint_rnnt_loss(
+        f, g, w, bias, labels, [T] * B, [U - 1] * B, V - 1, grad_costs=gc, big_blank_durations=big_blanks, sigma=sigma
+    )
+    ft, gt = torch.tensor(f, requires_grad=True), torch.tensor(g, requires_grad=True)
+    wt, bt = torch.tensor(w, requires_grad=True), torch.tensor(bias, requires_grad=True)
+    logits = torch.nn.functional.linear(torch.relu(ft[:, :, None, :] + gt[:, None, :, :]), wt, bt)
+    d_logits = []
+    for b in range(B):
+        nll, gl = multiblank_autograd(logits[b].detach().numpy(), labels[b], V - 1, big_blanks, sigma)
+        np.testing.assert_allclose(costs[b], nll, rtol=1e-10)
+        d_logits.append(gl * gc[b])
+    logits.backward(torch.tensor(np.stack(d_logits)))
+    for got, want in zip((d_f, d_g, d_w, d_b), (ft.grad, gt.grad, wt.grad, bt.grad)):
+        np.testing.assert_allclose(got, want.numpy(), rtol=1e-9, atol=1e-11)
