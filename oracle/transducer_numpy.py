@@ -16,18 +16,26 @@ How each function is pinned (tests/test_oracle_*.py):
   tdt_*             reference fixed vector (cost 4.155739 + 42 grads),
                     brute-force (token,duration) path enumeration,
                     torch autograd, T=1 and U=1 closed forms ......... pinned
-  tdt_* FastEmit    no reference vector exists; checked only against the
-                    sparse-posterior + softmax-Jacobian identity ..... derived
+  tdt_* FastEmit    PARITY UNPINNED: no reference vector or test exists for
+                    TDT with fastemit_lambda > 0; the terms are derived
+                    from gpu_rnnt_kernel.py:1353-1437 and checked only
+                    against their meaning (label-arc log-prob gradient
+                    x (1+lambda) through the token softmax Jacobian, the
+                    duration branch untouched) in torch autograd ..... derived
   multiblank_*      the reference holds no vector (its test compares two of
                     its own implementations on random input); with no big
                     blank and sigma = 0 it must give the RNNT golden vectors,
                     brute-force enumeration of every (token, blank-duration)
                     path, torch autograd of an alpha-only recursion,
                     llForward == beta(0,0) ........................... pinned
-  multiblank_* FastEmit  derived only, as for TDT
+  multiblank_* FastEmit  PARITY UNPINNED: derived only (gpu_rnnt_kernel.py:
+                    727-885), checked as for TDT
   joint_rnnt_loss   torch autograd (float64) through relu, linear and an
                     alpha-only recursion, with the bf16 roundings applied
-                    straight-through; the loss part is rnnt_loss above  pinned
+                    straight-through; the loss part is rnnt_loss above;
+                    with durations / big blanks: torch autograd of relu and
+                    linear fed with the logits-gradient of an independent
+                    alpha-only TDT / multi-blank recursion ............ pinned
   rnnt_logprobs*    torch log_softmax + gather (the reference's own etalon,
                     parts/k2/rnnt_logprobs.py:19-48) and torch autograd
                     through it, in float64 ........................... pinned
