@@ -373,7 +373,7 @@ int mi_transducer_describe_plan(int act_dtype, int B, int T, int U, int V, int D
   char denom[96], lattice[96], cells[48], grad[112];
   const BlockPlan dp = denom_block_plan(c);
   if (dp.RT) snprintf(denom, sizeof denom, "denom_block_kernel<%s, RT=%d, NVT=%d>", dt, dp.RT, dp.NVT);
-  else if (rows_R(c)) snprintf(denom, sizeof denom, "denom_rows_kernel<%s, R=%d, RPW=%d>", dt, rows_R(c), denom_rows_per_wave(rows_R(c)));
+  else if (denom_rows_R(c)) snprintf(denom, sizeof denom, "denom_rows_kernel<%s, R=%d, RPW=%d>", dt, denom_rows_R(c), denom_rows_per_wave(denom_rows_R(c)));
   else snprintf(denom, sizeof denom, "denom_gather_kernel<%s>", dt);
   const bool tdt = D > 0 && !use_plain_rnnt;
   const bool mb = num_big_blanks > 0;

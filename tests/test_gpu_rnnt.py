@@ -299,3 +299,25 @@ def test_loaded_library_is_the_in_tree_build():
 
     with open("/proc/self/maps") as f:
         assert any(_native.LIB_PATH in line for line in f)
+
+
+@pytest.mark.parametrize("V,dtype", [(520, torch.float32), (700, torch.float32), (1030, torch.float32), (1200, torch.float32),
+                                     (1400, torch.float32), (2056, torch.float32), (4104, torch.float32),
+                                     (8200, torch.float32), (1040, torch.bfloat16), (1500, torch.bfloat16),
+                                     (2060, torch.bfloat16), (2500, torch.bfloat16)])  # fmt: skip
+def test_vocabularies_just_past_a_power_of_two(V, dtype):
+    """Row lengths that take the in-between kernel shapes: 3, 5 or 6 vectors per lane in the denominator pass, a
+    third vector per thread in the gradient pass (e.g. 1024 tokens + blank + a few big blanks or durations)."""
+    rng = np.random.RandomState(V)
+    B, T, U = 2, 7, 5
+    x = torch.tensor(rng.randn(B, T, U, V), dtype=dtype)
+    labels = rng.randint(0, V - 1, size=(B, U - 1))
+    al, ll = np.array([T, 4]), np.array([2, U - 1])
+    acts = x.to(DEV).requires_grad_(True)
+    lab, ald, lld = to_dev(labels, al, ll)
+    costs = RNNTLossNumba(blank=V - 1, reduction='none', fastemit_lambda=0.01, clamp=0.3)(acts, lab, ald, lld)
+    costs.sum().backward()
+    c_ref, g_ref, _ = oracle.rnnt_loss(x.float().numpy(), labels, al, ll, V - 1, 0.01, 0.3)
+    f32 = dtype == torch.float32
+    np.testing.assert_allclose(costs.detach().float().cpu().numpy(), c_ref, rtol=1e-6 if f32 else 2.0**-7)
+    assert np.abs(acts.grad.float().cpu().numpy() - g_ref).max() < (2e-6 if f32 else 2.0**-8)

@@ -78,7 +78,10 @@ def test_kernel_plan_of_the_documented_shapes(built_lib):
     assert p["lattice"] == "rnnt_lattice_kernel<K=2>" and p["cells"] == "-"
     p = plan(F32, 16, 375, 121, 1028, num_big_blanks=3)  # multi-blank: three big blanks inside V
     assert p["lattice"] == "multiblank_lattice_kernel<NBC=4>" and p["cells"] == "multiblank_cell_kernel"
-    assert p["gradient"] == "grad_block_kernel<f32, RT=256, NVT=2, coef> + multiblank_fixup_kernel"
+    # 257 whole vectors, one past a power of two: 5 vectors per lane in pass 1, a third (nearly empty) vector per
+    # thread in the gradient pass rather than twice the threads
+    assert p["denominators"] == "denom_rows_kernel<f32, R=5, RPW=1>"
+    assert p["gradient"] == "grad_block_kernel<f32, RT=128, NVT=3, coef> + multiblank_fixup_kernel"
     p = plan(F32, 2, 50, 1024, 1028, max_duration=8, num_big_blanks=3)  # ring of 9 x 6 x 1024 doubles > 160 KB of LDS
     assert p["lattice"] == "multiblank_lattice_pull_kernel"
     p = plan(F32, 2, 50, 513, 1025, D=9, max_duration=8)  # beyond 256 label columns: a wave per direction
