@@ -10,7 +10,7 @@
  * Conventions
  *   - plain C: device pointers, sizes, a hipStream_t passed as void*; no torch types.
  *   - every function returns 0 on success, 1 on an invalid value (mirrors RNNTStatus,
- *     utils/global_constants.py:66-68), 2 if a HIP launch failed.  Nothing throws.
+ *     utils/global_constants.py:66-68), 2 if a HIP launch failed (3: see mi_rnnt_loss_static).  Nothing throws.
  *   - all work is enqueued on `stream`; no call blocks the host, allocates or frees.
  *   - all device memory is caller-owned.  `workspace` is scratch of at least
  *     mi_transducer_workspace_bytes() bytes, 256-byte aligned; its contents after a
@@ -39,6 +39,7 @@ extern "C" {
 #define MI_TRANSDUCER_SUCCESS 0
 #define MI_TRANSDUCER_INVALID_VALUE 1
 #define MI_TRANSDUCER_LAUNCH_FAILURE 2
+#define MI_TRANSDUCER_TOO_LARGE 3 /* mi_rnnt_loss_static only: the shape needs more than the built-in workspace */
 
 #define MI_DTYPE_F32 0
 #define MI_DTYPE_BF16 1
@@ -92,6 +93,24 @@ int mi_rnnt_loss(const void* acts, int act_dtype, const int64_t* labels, const i
                  int grad_scale_stride, float grad_mul, int B, int T, int U, int V, int blank, float fastemit_lambda,
                  float clamp, void* workspace, size_t workspace_bytes, void* stream);
 
+/* mi_rnnt_loss without a workspace argument, for callers that cannot allocate one: code under HIP graph capture,
+ * tight serving loops, harnesses that forbid hipMalloc.  It has no counterpart in the reference (whose wrapper
+ * allocates a workspace per call, rnnt.py:182-189).  The lattice state lives in a device array built into the
+ * library, MI_TRANSDUCER_STATIC_WORKSPACE_BYTES (64 MiB) per GPU that the library runs on, held until the process
+ * ends; a shape whose workspace (mi_transducer_workspace_bytes(B, T, U, 0)) is larger returns
+ * MI_TRANSDUCER_TOO_LARGE and launches nothing.  B=16, T=375, U=121 needs 50 MB.  The call itself allocates and
+ * frees nothing and does not block.  All calls on one GPU share that one array: two calls that overlap in time
+ * on the same GPU (different streams, or threads) race; calls on one stream are fine, and nothing has to be
+ * cleared between calls.  mi_transducer_init() looks the array's address up for the current device (the first
+ * mi_rnnt_loss_static on a device does it otherwise): call it once per device before capturing a graph.
+ * Results are those of mi_rnnt_loss, bit for bit. */
+#define MI_TRANSDUCER_STATIC_WORKSPACE_BYTES (64u << 20)
+int mi_transducer_init(void);
+int mi_rnnt_loss_static(const void* acts, int act_dtype, const int64_t* labels, const int64_t* act_lens,
+                        const int64_t* label_lens, float* costs, void* grads, const float* grad_scale,
+                        int grad_scale_stride, float grad_mul, int B, int T, int U, int V, int blank,
+                        float fastemit_lambda, float clamp, void* stream);
+
 /* TDT.  acts is the COMBINED tensor [B,T,U,V+D]: V token logits (blank included)
  * followed by D duration logits, exactly what TDTLossNumba.forward receives
  * (rnnt_pytorch.py:554-583); the split, the .contiguous() copies and the duration
@@ -119,6 +138,31 @@ int mi_tdt_loss(const void* acts, int act_dtype, const int64_t* labels, const in
                 float grad_mul, int B, int T, int U, int V, int D, const int32_t* durations_host, int blank,
                 float fastemit_lambda, float clamp, float sigma, int use_plain_rnnt, void* workspace,
                 size_t workspace_bytes, void* stream);
+
+/* TDT with the reference's function-level operands (tdt_loss_gpu, rnnt.py:239-255; GPUTDT.cost_and_grad /
+ * score_forward, utils/cuda_utils/gpu_rnnt.py:563-807): label_acts [B,T,U,V] raw token logits and duration_acts
+ * [B,T,U,D] duration LOG-PROBS (the caller has applied log_softmax, rnnt_pytorch.py:568) in two tensors of the
+ * same dtype.  label_grads [B,T,U,V] receives the gradient w.r.t. the token logits (as mi_tdt_backward's token
+ * block) and duration_grads [B,T,U,D] the gradient w.r.t. the duration log-probs, i.e. minus the posterior of the
+ * arcs of each duration (gpu_rnnt_kernel.py:1328-1341; no clamp, no FastEmit on these); padded cells get zeros in
+ * both.  use_plain_rnnt != 0 (the omega branch): plain RNNT on the token logits, duration_grads all zero.
+ * The workspace is mi_transducer_workspace_bytes(B, T, U, D).  In mi_tdt_split_loss both gradient pointers are
+ * given or both are NULL (forward only). */
+int mi_tdt_split_forward(const void* label_acts, const void* duration_acts, int act_dtype, const int64_t* labels,
+                         const int64_t* act_lens, const int64_t* label_lens, float* costs, int B, int T, int U, int V,
+                         int D, const int32_t* durations_host, int blank, float fastemit_lambda, float sigma,
+                         int use_plain_rnnt, int with_betas, void* workspace, size_t workspace_bytes, void* stream);
+int mi_tdt_split_backward(const void* label_acts, int act_dtype, const int64_t* labels, const int64_t* act_lens,
+                          const int64_t* label_lens, void* label_grads, void* duration_grads,
+                          const float* grad_scale, int grad_scale_stride, float grad_mul, int B, int T, int U, int V,
+                          int D, const int32_t* durations_host, int blank, float fastemit_lambda, float clamp,
+                          float sigma, int use_plain_rnnt, void* workspace, size_t workspace_bytes, void* stream);
+int mi_tdt_split_loss(const void* label_acts, const void* duration_acts, int act_dtype, const int64_t* labels,
+                      const int64_t* act_lens, const int64_t* label_lens, float* costs, void* label_grads,
+                      void* duration_grads, const float* grad_scale, int grad_scale_stride, float grad_mul, int B,
+                      int T, int U, int V, int D, const int32_t* durations_host, int blank, float fastemit_lambda,
+                      float clamp, float sigma, int use_plain_rnnt, void* workspace, size_t workspace_bytes,
+                      void* stream);
 
 /* ---- multi-blank transducer ---------------------------------------------------------
  * Replaces rnnt.py:366-483 (multiblank_rnnt_loss_gpu) and what it drives:

@@ -16,8 +16,9 @@ INCLUDE_DIR = os.path.join(os.path.dirname(_HERE), "include")
 LIB_PATH = os.environ.get("MI_TRANSDUCER_LIB") or os.path.join(CSRC_DIR, "libmi_transducer.so")
 SOURCES = [os.path.join(CSRC_DIR, "mi_transducer.hip")]
 
-ABI_VERSION = 13
-SUCCESS, INVALID_VALUE, LAUNCH_FAILURE = 0, 1, 2
+ABI_VERSION = 14
+SUCCESS, INVALID_VALUE, LAUNCH_FAILURE, TOO_LARGE = 0, 1, 2, 3
+STATIC_WORKSPACE_BYTES = 64 << 20
 DTYPE_F32, DTYPE_BF16, DTYPE_F16 = 0, 1, 2
 
 HIPCC_FLAGS = [
@@ -61,12 +62,21 @@ _SIGNATURES = {
                          _c_int, _c_int, _c_float, _c_float, _vp, _c_size_t, _vp],
     "mi_rnnt_loss": [_vp, _c_int, _vp, _vp, _vp, _vp, _vp, _vp, _c_int, _c_float, _c_int, _c_int, _c_int, _c_int,
                      _c_int, _c_float, _c_float, _vp, _c_size_t, _vp],
+    "mi_transducer_init": [],
+    "mi_rnnt_loss_static": [_vp, _c_int, _vp, _vp, _vp, _vp, _vp, _vp, _c_int, _c_float, _c_int, _c_int, _c_int, _c_int,
+                            _c_int, _c_float, _c_float, _vp],
     "mi_tdt_forward": [_vp, _c_int, _vp, _vp, _vp, _vp, _c_int, _c_int, _c_int, _c_int, _c_int, _vp, _c_int, _c_float,
                        _c_float, _c_int, _c_int, _vp, _c_size_t, _vp],
     "mi_tdt_backward": [_vp, _c_int, _vp, _vp, _vp, _vp, _vp, _c_int, _c_float, _c_int, _c_int, _c_int, _c_int,
                         _c_int, _c_int, _vp, _c_int, _c_float, _c_float, _c_float, _c_int, _vp, _c_size_t, _vp],
     "mi_tdt_loss": [_vp, _c_int, _vp, _vp, _vp, _vp, _vp, _vp, _c_int, _c_float, _c_int, _c_int, _c_int, _c_int,
                     _c_int, _vp, _c_int, _c_float, _c_float, _c_float, _c_int, _vp, _c_size_t, _vp],
+    "mi_tdt_split_forward": [_vp, _vp, _c_int, _vp, _vp, _vp, _vp, _c_int, _c_int, _c_int, _c_int, _c_int, _vp, _c_int,
+                             _c_float, _c_float, _c_int, _c_int, _vp, _c_size_t, _vp],
+    "mi_tdt_split_backward": [_vp, _c_int, _vp, _vp, _vp, _vp, _vp, _vp, _c_int, _c_float, _c_int, _c_int, _c_int,
+                              _c_int, _c_int, _vp, _c_int, _c_float, _c_float, _c_float, _c_int, _vp, _c_size_t, _vp],
+    "mi_tdt_split_loss": [_vp, _vp, _c_int, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _c_int, _c_float, _c_int, _c_int, _c_int,
+                          _c_int, _c_int, _vp, _c_int, _c_float, _c_float, _c_float, _c_int, _vp, _c_size_t, _vp],
     "mi_multiblank_forward": [_vp, _c_int, _vp, _vp, _vp, _vp, _c_int, _c_int, _c_int, _c_int, _c_int, _vp, _c_int,
                               _c_float, _c_float, _c_int, _vp, _c_size_t, _vp],
     "mi_multiblank_backward": [_vp, _c_int, _vp, _vp, _vp, _vp, _vp, _c_int, _c_float, _c_int, _c_int, _c_int, _c_int,
@@ -149,6 +159,11 @@ def check_status(status, what):
         return
     if status == INVALID_VALUE:
         raise RuntimeError(f"{what}: invalid value passed to the transducer-loss library")
+    if status == TOO_LARGE:
+        raise RuntimeError(
+            f"{what}: the shape needs more than the {STATIC_WORKSPACE_BYTES >> 20} MiB workspace built into the "
+            "library; use the entry point that takes a caller-owned workspace"
+        )
     raise RuntimeError(f"{what}: HIP kernel launch failed (status {status})")
 
 

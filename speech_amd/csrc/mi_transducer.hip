@@ -25,6 +25,7 @@
 #include <stdio.h>
 #include <stdint.h>
 
+#include <mutex>
 #include <type_traits>
 #include <vector>
 
@@ -60,7 +61,7 @@ namespace {
 // ----------------------------------------------------------------------------------------
 extern "C" {
 
-int mi_transducer_abi_version(void) { return 13; }
+int mi_transducer_abi_version(void) { return 14; }
 
 int mi_transducer_workspace_bytes(int B, int T, int U, int D, size_t* out_bytes) {
   Layout L;
@@ -105,6 +106,57 @@ int mi_rnnt_loss(const void* acts, int act_dtype, const int64_t* labels, const i
   if (st || !grads) return st;
   return mi_rnnt_backward(acts, act_dtype, labels, act_lens, label_lens, grads, grad_scale, grad_scale_stride,
                           grad_mul, 0, B, T, U, V, blank, fastemit_lambda, clamp, workspace, workspace_bytes, stream);
+}
+
+// ----------------------------------------------------------------------------------------
+// The one entry point that brings its own workspace: a device array that lives in the code object.
+// ----------------------------------------------------------------------------------------
+}  // extern "C"
+
+static __device__ __align__(256) unsigned char scratch[MI_TRANSDUCER_STATIC_WORKSPACE_BYTES];
+
+namespace {
+constexpr int kMaxDevices = 64;
+void* g_scratch_ptr[kMaxDevices];  // per device: where that device holds its copy of `scratch`
+std::mutex g_scratch_mutex;
+
+// The address of `scratch` on the current device.  In host code the array's name is only a handle for the
+// runtime, never a device address: the address comes from hipGetSymbolAddress, once per device.
+int static_workspace(void** out) {
+  int dev = -1;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) return MI_TRANSDUCER_LAUNCH_FAILURE;
+  std::lock_guard<std::mutex> lock(g_scratch_mutex);
+  if (!g_scratch_ptr[dev]) {
+    void* p = nullptr;
+    if (hipGetSymbolAddress(&p, HIP_SYMBOL(scratch)) != hipSuccess || !p) return MI_TRANSDUCER_LAUNCH_FAILURE;
+    g_scratch_ptr[dev] = p;
+  }
+  *out = g_scratch_ptr[dev];
+  return MI_TRANSDUCER_SUCCESS;
+}
+}  // namespace
+
+extern "C" {
+
+int mi_transducer_init(void) {
+  void* p;
+  return static_workspace(&p);
+}
+
+int mi_rnnt_loss_static(const void* acts, int act_dtype, const int64_t* labels, const int64_t* act_lens,
+                        const int64_t* label_lens, float* costs, void* grads, const float* grad_scale,
+                        int grad_scale_stride, float grad_mul, int B, int T, int U, int V, int blank,
+                        float fastemit_lambda, float clamp, void* stream) {
+  Layout L;
+  if (!make_layout(B, T, U, 0, &L)) return MI_TRANSDUCER_INVALID_VALUE;
+  if (L.total > (size_t)MI_TRANSDUCER_STATIC_WORKSPACE_BYTES) return MI_TRANSDUCER_TOO_LARGE;
+  void* ws = nullptr;
+  const int st = static_workspace(&ws);
+  if (st) return st;
+  // nothing in the workspace has to start at zero: every kernel writes what later kernels of the call read, and
+  // what is left there by an earlier call is never read
+  return mi_rnnt_loss(acts, act_dtype, labels, act_lens, label_lens, costs, grads, grad_scale, grad_scale_stride,
+                      grad_mul, B, T, U, V, blank, fastemit_lambda, clamp, ws, L.total, stream);
 }
 
 int mi_tdt_forward(const void* acts, int act_dtype, const int64_t* labels, const int64_t* act_lens,
@@ -160,6 +212,65 @@ int mi_tdt_loss(const void* acts, int act_dtype, const int64_t* labels, const in
   return mi_tdt_backward(acts, act_dtype, labels, act_lens, label_lens, grads, grad_scale, grad_scale_stride, grad_mul,
                          0, B, T, U, V, D, durations_host, blank, fastemit_lambda, clamp, sigma, use_plain_rnnt,
                          workspace, workspace_bytes, stream);
+}
+
+int mi_tdt_split_forward(const void* label_acts, const void* duration_acts, int act_dtype, const int64_t* labels,
+                         const int64_t* act_lens, const int64_t* label_lens, float* costs, int B, int T, int U, int V,
+                         int D, const int32_t* durations_host, int blank, float fastemit_lambda, float sigma,
+                         int use_plain_rnnt, int with_betas, void* workspace, size_t workspace_bytes, void* stream) {
+  Common c;
+  TdtParams prm;
+  if (!costs || !duration_acts) return MI_TRANSDUCER_INVALID_VALUE;
+  int st = make_tdt_params(D, durations_host, sigma, &prm);
+  if (st) return st;
+  st = check_common(label_acts, act_dtype, labels, act_lens, label_lens, B, T, U, V, 0, blank, workspace,
+                    workspace_bytes, stream, &c, 0, D);
+  if (st) return st;
+  if ((st = run_denom(c))) return st;
+  if (use_plain_rnnt) return run_rnnt_lattice(c, costs, fastemit_lambda, with_betas);
+  if ((st = run_tdt_duration_planes(c, duration_acts, D))) return st;
+  return run_tdt_lattice(c, costs, fastemit_lambda, with_betas, prm);
+}
+
+int mi_tdt_split_backward(const void* label_acts, int act_dtype, const int64_t* labels, const int64_t* act_lens,
+                          const int64_t* label_lens, void* label_grads, void* duration_grads,
+                          const float* grad_scale, int grad_scale_stride, float grad_mul, int B, int T, int U, int V,
+                          int D, const int32_t* durations_host, int blank, float fastemit_lambda, float clamp,
+                          float sigma, int use_plain_rnnt, void* workspace, size_t workspace_bytes, void* stream) {
+  Common c;
+  TdtParams prm;
+  if (!label_grads || !duration_grads || clamp < 0.f || grad_scale_stride < 0) return MI_TRANSDUCER_INVALID_VALUE;
+  int st = make_tdt_params(D, durations_host, sigma, &prm);
+  if (st) return st;
+  st = check_common(label_acts, act_dtype, labels, act_lens, label_lens, B, T, U, V, 0, blank, workspace,
+                    workspace_bytes, stream, &c, 0, D);
+  if (st) return st;
+  const ScaleArg sc = {grad_scale, grad_scale_stride, grad_mul};
+  if (use_plain_rnnt) {  // gpu_rnnt.py:646-682: token gradient from the RNNT kernel, duration gradient stays zero
+    const bool fused = rnnt_rows_fused(c, label_grads);
+    if (!fused && (st = run_rnnt_cells(c, sc, fastemit_lambda, clamp))) return st;
+    if ((st = run_grad_stream(c, label_grads, 0, fused, sc, fastemit_lambda, clamp))) return st;
+    return run_tdt_duration_grads(c, duration_grads, D, 1);
+  }
+  if ((st = run_tdt_cells(c, sc, fastemit_lambda, clamp, prm, 1))) return st;
+  if ((st = run_grad_stream(c, label_grads, 0, false, sc, fastemit_lambda, clamp))) return st;
+  return run_tdt_duration_grads(c, duration_grads, D, 0);
+}
+
+int mi_tdt_split_loss(const void* label_acts, const void* duration_acts, int act_dtype, const int64_t* labels,
+                      const int64_t* act_lens, const int64_t* label_lens, float* costs, void* label_grads,
+                      void* duration_grads, const float* grad_scale, int grad_scale_stride, float grad_mul, int B,
+                      int T, int U, int V, int D, const int32_t* durations_host, int blank, float fastemit_lambda,
+                      float clamp, float sigma, int use_plain_rnnt, void* workspace, size_t workspace_bytes,
+                      void* stream) {
+  if ((label_grads == nullptr) != (duration_grads == nullptr)) return MI_TRANSDUCER_INVALID_VALUE;
+  int st = mi_tdt_split_forward(label_acts, duration_acts, act_dtype, labels, act_lens, label_lens, costs, B, T, U, V, D,
+                                durations_host, blank, fastemit_lambda, sigma, use_plain_rnnt, label_grads != nullptr,
+                                workspace, workspace_bytes, stream);
+  if (st || !label_grads) return st;
+  return mi_tdt_split_backward(label_acts, act_dtype, labels, act_lens, label_lens, label_grads, duration_grads,
+                               grad_scale, grad_scale_stride, grad_mul, B, T, U, V, D, durations_host, blank,
+                               fastemit_lambda, clamp, sigma, use_plain_rnnt, workspace, workspace_bytes, stream);
 }
 
 int mi_multiblank_forward(const void* acts, int act_dtype, const int64_t* labels, const int64_t* act_lens,

@@ -15,6 +15,7 @@ backward recomputes).  bfloat16 / float16 logits are read natively, arithmetic i
 import torch
 
 from speech_amd import _native
+from speech_amd.rnnt_loss.rnnt_pytorch import grads_like
 from speech_amd.rnnt_loss.rnnt import _dtype_code, _labels_ptr, _ptr, _require_gpu, _stream, new_workspace
 
 __all__ = ["RnntLogProbs", "rnnt_logprobs", "rnnt_logprobs_triton"]
@@ -67,7 +68,7 @@ class RnntLogProbs(torch.autograd.Function):
             workspace, have_state = new_workspace(logits), 0
         grad_target_scores = grad_target_scores.to(torch.float32).contiguous()
         grad_blank_scores = grad_blank_scores.to(torch.float32).contiguous()
-        grad_logits = torch.empty_like(logits)  # every element is written, padded cells as zeros
+        grad_logits = grads_like(logits)  # every element is written, padded cells as zeros
         with torch.cuda.device(device):
             status = _native.lib().mi_rnnt_logprobs_backward(
                 _ptr(logits), _dtype_code(logits), _labels_ptr(targets), _ptr(source_lengths), _ptr(target_lengths),

@@ -1,4 +1,4 @@
-from speech_amd.rnnt_loss.rnnt import multiblank_rnnt_loss_gpu, rnnt_loss_gpu, tdt_loss_gpu
+from speech_amd.rnnt_loss.rnnt import combined_tdt_loss_gpu, multiblank_rnnt_loss_gpu, rnnt_loss_gpu, tdt_loss_gpu
 from speech_amd.rnnt_loss.rnnt_pytorch import (
     MultiblankRNNTLossMI355X,
     MultiblankRNNTLossNumba,
@@ -12,6 +12,7 @@ from speech_amd.rnnt_loss.rnnt_pytorch import (
 __all__ = [
     'rnnt_loss_gpu',
     'tdt_loss_gpu',
+    'combined_tdt_loss_gpu',
     'multiblank_rnnt_loss_gpu',
     'RNNTLossNumba',
     'TDTLossNumba',

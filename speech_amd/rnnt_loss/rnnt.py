@@ -11,13 +11,16 @@ folded in, instead of being stored in forward and rescaled later.
 Differences a caller can see:
   * nothing blocks the host (the reference ends with stream.synchronize(),
     utils/cuda_utils/gpu_rnnt.py:229);
-  * `tdt_loss_gpu` takes the combined [B,T,U,V+D] logits and returns the
-    gradient w.r.t. them (the kernels do the split and the duration
-    log-softmax that TDTLossNumba.forward does with torch ops, rnnt_pytorch.py:564-568);
-  * there is no CPU implementation here: CPU tensors raise.
+  * besides `tdt_loss_gpu` (the reference's operands: token logits and
+    duration log-probs in two tensors) there is `combined_tdt_loss_gpu`, which
+    takes the combined [B,T,U,V+D] logits and returns the gradient w.r.t. them
+    (the kernels do the split and the duration log-softmax that
+    TDTLossNumba.forward does with torch ops, rnnt_pytorch.py:564-568);
+  * these functions run on the GPU only (the module-level RNNT loss has a CPU path of its own).
 """
 
 import ctypes
+import random
 
 import torch
 
@@ -268,12 +271,73 @@ def rnnt_loss_gpu(
 
 
 def tdt_loss_gpu(
+    label_acts, duration_acts, labels, input_lengths, label_lengths, costs, label_grads, duration_grads, blank_label,
+    durations, fastemit_lambda, clamp, num_threads, sigma, omega,
+):  # fmt: skip
+    """Drop-in for rnnt.py:239-363, argument for argument: label_acts [B,T,U,V] are raw token logits,
+    duration_acts [B,T,U,D] duration log-probs; costs [B], label_grads [B,T,U,V] (gradient w.r.t. the token
+    logits) and duration_grads [B,T,U,D] (gradient w.r.t. the duration log-probs, gpu_rnnt_kernel.py:1328-1341) are
+    filled in place; label_grads None means forward only (rnnt.py:336-345).  With probability omega the call takes
+    the plain RNNT kernels and leaves duration_grads zero; the draw is random.uniform(0, 1) as in gpu_rnnt.py:606.
+    costs may be float32 or, as the reference allocates it (rnnt_pytorch.py:145), of the dtype of the logits."""
+    del num_threads
+    _require_gpu(label_acts, "tdt_loss_gpu")
+    if label_acts.dtype != duration_acts.dtype or label_acts.shape[:3] != duration_acts.shape[:3]:
+        raise ValueError("label_acts and duration_acts must share dtype and their first three dimensions")
+    if not (label_acts.is_contiguous() and duration_acts.is_contiguous()):
+        raise ValueError("label_acts and duration_acts must be contiguous")
+    B, T, U, V = label_acts.shape
+    D = len(durations)
+    if duration_acts.shape[3] != D:
+        raise ValueError(f"duration_acts must hold {D} entries per cell, got {duration_acts.shape[3]}")
+    if (label_grads is None) != (duration_grads is None):
+        raise ValueError("label_grads and duration_grads are given together or not at all")
+    workspace = new_workspace(label_acts, D)
+    costs32 = costs if costs.dtype == torch.float32 else torch.empty(B, dtype=torch.float32, device=costs.device)
+    use_plain_rnnt = random.uniform(0, 1) < omega
+    keep, dur_ptr = _durations_array(durations)
+    with torch.cuda.device(label_acts.device):
+        status = _native.lib().mi_tdt_split_loss(
+            _ptr(label_acts), _ptr(duration_acts), _dtype_code(label_acts), _labels_ptr(labels), _ptr(input_lengths),
+            _ptr(label_lengths), _ptr(costs32), _ptr(label_grads), _ptr(duration_grads), None, 0, 1.0, B, T, U, V, D,
+            dur_ptr, int(blank_label), float(fastemit_lambda), float(clamp), float(sigma), int(use_plain_rnnt),
+            _ptr(workspace), workspace.numel(), _stream(label_acts.device),
+        )  # fmt: skip
+    del keep
+    _native.check_status(status, "Could not calculate forward scores")
+    if costs32 is not costs:
+        costs.copy_(costs32)
+    return True
+
+
+def rnnt_loss_static(acts, labels, input_lengths, label_lengths, costs, grads, blank_label, fastemit_lambda, clamp):
+    """rnnt_loss_gpu for callers that must not allocate (HIP graph capture, serving loops): same results, but the
+    lattice state lives in a 64 MiB device array built into the library instead of a workspace tensor, so this
+    function creates no tensor at all.  Shapes whose workspace is larger raise RuntimeError.  Calls on one GPU
+    share that array: they must not overlap in time (one stream, or the caller orders them)."""
+    _require_gpu(acts, "rnnt_loss_static")
+    B, T, U, V = acts.shape
+    if costs.dtype != torch.float32:
+        raise TypeError("costs must be float32")
+    with torch.cuda.device(acts.device):
+        status = _native.lib().mi_rnnt_loss_static(
+            _ptr(acts), _dtype_code(acts), _labels_ptr(labels), _ptr(input_lengths), _ptr(label_lengths), _ptr(costs),
+            _ptr(grads), None, 0, 1.0, B, T, U, V, int(blank_label), float(fastemit_lambda), float(clamp),
+            _stream(acts.device),
+        )  # fmt: skip
+    _native.check_status(status, "rnnt_loss_static")
+    return True
+
+
+def combined_tdt_loss_gpu(
     acts, labels, input_lengths, label_lengths, costs, grads, blank_label, durations, fastemit_lambda, clamp,
     num_threads=0, sigma=0.0, use_plain_rnnt=False,
 ):  # fmt: skip
-    """TDT counterpart (rnnt.py:239-363) on the combined [B,T,U,V+D] logits; costs is float32 [B]."""
+    """TDT on the COMBINED [B,T,U,V+D] logits (what TDTLossNumba.forward receives, rnnt_pytorch.py:554-583): the
+    split, the duration log_softmax and its backward happen in the kernels, and grads is w.r.t. the combined
+    logits.  costs is float32 [B].  The caller decides the omega branch (use_plain_rnnt)."""
     del num_threads
-    _require_gpu(acts, "tdt_loss_gpu")
+    _require_gpu(acts, "combined_tdt_loss_gpu")
     B, T, U, VD = acts.shape
     D = len(durations)
     workspace = new_workspace(acts, D)

@@ -70,6 +70,19 @@ def _start_padding_fill(grads, act_lens, label_lens):
     return done
 
 
+def grads_like(acts):
+    """An uninitialised tensor of the shape and dtype of acts whose storage starts at the same offset within a
+    16-byte line as acts does.  The gradient pass stores whole 16-byte vectors where the logits row has them, which
+    needs the two buffers in phase; a fresh allocation is 16-byte aligned, a view such as `big[1:]` need not be."""
+    phase = acts.data_ptr() & 15
+    if phase == 0:
+        return torch.empty_like(acts)
+    size = acts.element_size()
+    flat = torch.empty(acts.numel() + 16 // size, dtype=acts.dtype, device=acts.device)
+    first = ((phase - flat.data_ptr()) & 15) // size
+    return flat[first : first + acts.numel()].view(acts.shape)
+
+
 def check_type(var, t, name):
     if var.dtype is not t:
         raise TypeError("{} must be {}".format(name, t))
@@ -136,9 +149,16 @@ class _PendingLengthCheck:
             self.host = torch.stack([torch.max(lengths), torch.max(label_lengths)])
             self.event = None
 
-    def finish(self):
+    def drain(self):
+        """Wait for the kernel that writes into the pinned buffer, so that the buffer is not handed back to the host
+        allocator (and on to some other user) while that write is still queued.  For the error paths that drop
+        this object without finish()."""
         if self.event is not None:
             self.event.synchronize()
+            self.event = None
+
+    def finish(self):
+        self.drain()
         max_T, max_U = int(self.host[0]), int(self.host[1])
         if self.T < max_T if self.padded_T else self.T != max_T:
             raise ValueError(f"Input length mismatch! Given T: {self.T}, Expected max T from input lengths: {max_T}")
@@ -227,20 +247,23 @@ class _RNNTNumba(Function):
             )
         _check_same_device(acts, labels, act_lens, label_lens)
         pending = _PendingLengthCheck(acts, act_lens, label_lens)
-
-        need_grad = ctx.needs_input_grad[0]
-        batch = acts.size(0)
-        costs = torch.empty(batch, device=acts.device, dtype=torch.float32)
-        workspace = rnnt.new_workspace(acts)
-        ctx.padding = None
-        if need_grad and OVERLAP_PADDING:
-            grads = torch.empty_like(acts)
-            rnnt.denominators(acts, labels, act_lens, label_lens, blank, workspace)
-            ctx.padding = (grads, _start_padding_fill(grads, act_lens, label_lens))
-            B, T, U = acts.shape[:3]
-            rnnt.rnnt_lattice(act_lens, label_lens, costs, B, T, U, fastemit_lambda, True, workspace)
-        else:
-            rnnt.rnnt_forward(acts, labels, act_lens, label_lens, costs, blank, fastemit_lambda, need_grad, workspace)
+        try:
+            need_grad = ctx.needs_input_grad[0]
+            batch = acts.size(0)
+            costs = torch.empty(batch, device=acts.device, dtype=torch.float32)
+            workspace = rnnt.new_workspace(acts)
+            ctx.padding = None
+            if need_grad and OVERLAP_PADDING:
+                grads = grads_like(acts)
+                rnnt.denominators(acts, labels, act_lens, label_lens, blank, workspace)
+                ctx.padding = (grads, _start_padding_fill(grads, act_lens, label_lens))
+                B, T, U = acts.shape[:3]
+                rnnt.rnnt_lattice(act_lens, label_lens, costs, B, T, U, fastemit_lambda, True, workspace)
+            else:
+                rnnt.rnnt_forward(acts, labels, act_lens, label_lens, costs, blank, fastemit_lambda, need_grad, workspace)
+        except BaseException:
+            pending.drain()  # the pinned buffer must outlive the kernel that writes into it
+            raise
         pending.finish()  # raises ValueError exactly where certify_inputs would
 
         costs = _reduce_costs(costs, reduction, batch)
@@ -254,7 +277,7 @@ class _RNNTNumba(Function):
         acts, labels, act_lens, label_lens, workspace = ctx.saved_tensors
         blank, reduction, fastemit_lambda, clamp = ctx.params
         prepared, ctx.padding = ctx.padding, None  # the prepared buffer serves the first backward call only
-        grads = prepared[0] if prepared else torch.empty_like(acts)
+        grads = prepared[0] if prepared else grads_like(acts)
         scale, stride, mul = _grad_scale(grad_output, reduction, acts.size(0), acts.device)
         rnnt.rnnt_backward(
             acts, labels, act_lens, label_lens, grads, scale, blank, fastemit_lambda, clamp, workspace, stride, mul,
@@ -283,29 +306,32 @@ class _TDTNumba(Function):
         if acts.shape[-1] <= len(durations):
             raise ValueError("acts must hold the token logits followed by one logit per duration")
         pending = _PendingLengthCheck(acts, act_lens, label_lens)
-
-        need_grad = ctx.needs_input_grad[0]
-        batch = acts.size(0)
-        costs = torch.empty(batch, device=acts.device, dtype=torch.float32)
-        workspace = rnnt.new_workspace(acts, len(durations))
-        # gpu_rnnt.py:606-607: one host-side draw per call decides between the TDT and the plain RNNT kernels
-        use_plain_rnnt = random.uniform(0, 1) < omega
-        ctx.padding = None
-        if need_grad and OVERLAP_PADDING:
-            grads = torch.empty_like(acts)
-            D = len(durations)
-            rnnt.denominators(acts, labels, act_lens, label_lens, blank, workspace, D)
-            ctx.padding = (grads, _start_padding_fill(grads, act_lens, label_lens))
-            B, T, U = acts.shape[:3]
-            if use_plain_rnnt:
-                rnnt.rnnt_lattice(act_lens, label_lens, costs, B, T, U, fastemit_lambda, True, workspace, D)
+        try:
+            need_grad = ctx.needs_input_grad[0]
+            batch = acts.size(0)
+            costs = torch.empty(batch, device=acts.device, dtype=torch.float32)
+            workspace = rnnt.new_workspace(acts, len(durations))
+            # gpu_rnnt.py:606-607: one host-side draw per call decides between the TDT and the plain RNNT kernels
+            use_plain_rnnt = random.uniform(0, 1) < omega
+            ctx.padding = None
+            if need_grad and OVERLAP_PADDING:
+                grads = grads_like(acts)
+                D = len(durations)
+                rnnt.denominators(acts, labels, act_lens, label_lens, blank, workspace, D)
+                ctx.padding = (grads, _start_padding_fill(grads, act_lens, label_lens))
+                B, T, U = acts.shape[:3]
+                if use_plain_rnnt:
+                    rnnt.rnnt_lattice(act_lens, label_lens, costs, B, T, U, fastemit_lambda, True, workspace, D)
+                else:
+                    rnnt.tdt_lattice(act_lens, label_lens, costs, B, T, U, durations, fastemit_lambda, sigma, True, workspace)
             else:
-                rnnt.tdt_lattice(act_lens, label_lens, costs, B, T, U, durations, fastemit_lambda, sigma, True, workspace)
-        else:
-            rnnt.tdt_forward(
-                acts, labels, act_lens, label_lens, costs, blank, durations, fastemit_lambda, sigma, use_plain_rnnt,
-                need_grad, workspace,
-            )  # fmt: skip
+                rnnt.tdt_forward(
+                    acts, labels, act_lens, label_lens, costs, blank, durations, fastemit_lambda, sigma, use_plain_rnnt,
+                    need_grad, workspace,
+                )  # fmt: skip
+        except BaseException:
+            pending.drain()  # the pinned buffer must outlive the kernel that writes into it
+            raise
         pending.finish()
 
         # the reference allocates TDT costs in the dtype of acts (rnnt_pytorch.py:145)
@@ -322,7 +348,7 @@ class _TDTNumba(Function):
         acts, labels, act_lens, label_lens, workspace = ctx.saved_tensors
         blank, durations, reduction, fastemit_lambda, clamp, sigma, use_plain_rnnt = ctx.params
         prepared, ctx.padding = ctx.padding, None
-        grads = prepared[0] if prepared else torch.empty_like(acts)
+        grads = prepared[0] if prepared else grads_like(acts)
         scale, stride, mul = _grad_scale(grad_output, reduction, acts.size(0), acts.device)
         rnnt.tdt_backward(
             acts, labels, act_lens, label_lens, grads, scale, blank, durations, fastemit_lambda, clamp, sigma,
@@ -350,14 +376,17 @@ class _MultiblankRNNTNumba(Function):
         if blank - len(durations) < 0 or blank >= acts.shape[-1]:
             raise ValueError("the big blanks sit at blank-1-i: blank must leave room for them below it")
         pending = _PendingLengthCheck(acts, act_lens, label_lens)
-
-        need_grad = ctx.needs_input_grad[0]
-        batch = acts.size(0)
-        costs = torch.empty(batch, device=acts.device, dtype=torch.float32)
-        workspace = rnnt.new_workspace(acts, len(durations))
-        rnnt.multiblank_forward(
-            acts, labels, act_lens, label_lens, costs, blank, durations, fastemit_lambda, sigma, need_grad, workspace
-        )
+        try:
+            need_grad = ctx.needs_input_grad[0]
+            batch = acts.size(0)
+            costs = torch.empty(batch, device=acts.device, dtype=torch.float32)
+            workspace = rnnt.new_workspace(acts, len(durations))
+            rnnt.multiblank_forward(
+                acts, labels, act_lens, label_lens, costs, blank, durations, fastemit_lambda, sigma, need_grad, workspace
+            )
+        except BaseException:
+            pending.drain()  # the pinned buffer must outlive the kernel that writes into it
+            raise
         pending.finish()
 
         # the reference allocates these costs in the dtype of acts (rnnt_pytorch.py:232)
@@ -373,7 +402,7 @@ class _MultiblankRNNTNumba(Function):
     def backward(ctx, grad_output):
         acts, labels, act_lens, label_lens, workspace = ctx.saved_tensors
         blank, durations, reduction, fastemit_lambda, clamp, sigma = ctx.params
-        grads = torch.empty_like(acts)
+        grads = grads_like(acts)
         scale, stride, mul = _grad_scale(grad_output, reduction, acts.size(0), acts.device)
         rnnt.multiblank_backward(
             acts, labels, act_lens, label_lens, grads, scale, blank, durations, fastemit_lambda, clamp, sigma,

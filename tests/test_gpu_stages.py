@@ -51,23 +51,89 @@ def test_denominators_then_lattice_is_the_forward_call(with_betas):
     np.testing.assert_allclose(split.cpu().numpy(), c_ref, rtol=1e-6)
 
 
-def test_tdt_function_level_seam():
+def test_combined_tdt_function_level_seam():
     B, T, U, V, durations = 3, 9, 5, 12, [0, 1, 2, 3]
     x, labels, al, ll = make(3, B, T, U, V + len(durations))
     acts = torch.tensor(x, device=DEV)
     lab, ald, lld = to_dev(labels, al, ll)
     costs = torch.zeros(B, device=DEV)
     grads = torch.full_like(acts, float('nan'))
-    assert rnnt.tdt_loss_gpu(acts, lab, ald, lld, costs, grads, V - 1, durations, 0.01, 0.2, 0, 0.05) is True
+    assert rnnt.combined_tdt_loss_gpu(acts, lab, ald, lld, costs, grads, V - 1, durations, 0.01, 0.2, 0, 0.05) is True
     c_ref, g_ref, _ = oracle.tdt_loss(x, labels, al, ll, V - 1, durations, 0.05, 0.01, 0.2)
     np.testing.assert_allclose(costs.cpu().numpy(), c_ref, rtol=1e-6)
     assert np.abs(grads.cpu().numpy() - g_ref).max() < 2e-6
     # grads None: forward only (rnnt.py:336-345)
     only = torch.zeros(B, device=DEV)
-    assert rnnt.tdt_loss_gpu(acts, lab, ald, lld, only, None, V - 1, durations, 0.01, 0.2, 0, 0.05) is True
+    assert rnnt.combined_tdt_loss_gpu(acts, lab, ald, lld, only, None, V - 1, durations, 0.01, 0.2, 0, 0.05) is True
     assert torch.equal(only, costs)
     with pytest.raises(TypeError):
-        rnnt.tdt_loss_gpu(acts, lab, ald, lld, costs.double(), None, V - 1, durations, 0.0, 0.0, 0, 0.0)
+        rnnt.combined_tdt_loss_gpu(acts, lab, ald, lld, costs.double(), None, V - 1, durations, 0.0, 0.0, 0, 0.0)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("V", [12, 300, 1025])
+def test_tdt_loss_gpu_with_the_reference_operands(dtype, V):
+    """tdt_loss_gpu driven the way _TDTNumba.forward drives it (rnnt_pytorch.py:101-196): the caller splits the
+    combined tensor, log-softmaxes the duration part and owns zero-filled costs / label_grads / duration_grads.
+    label_grads is the gradient w.r.t. the token logits, duration_grads w.r.t. the duration LOG-PROBS
+    (gpu_rnnt_kernel.py:1328-1341): both against the oracle's tdt_grads, which keeps them apart."""
+    import random
+
+    B, T, U, durations, sigma, lam, clamp = 3, 9, 5, [0, 1, 2, 3], 0.05, 0.01, 0.2
+    D = len(durations)
+    x, labels, al, ll = make(V, B, T, U, V + D)
+    x = torch.tensor(x, dtype=dtype)
+    lab, ald, lld = to_dev(labels, al, ll)
+    label_acts = x[..., :V].contiguous().to(DEV)
+    # the duration log-probs the kernels see are the caller's, rounded to the dtype of the logits
+    duration_acts = torch.nn.functional.log_softmax(x[..., V:].float(), dim=-1).to(dtype).contiguous().to(DEV)
+    # the oracle's per-utterance functions take log-probs for both parts, so they see exactly the (rounded,
+    # hence not exactly normalised) duration log-probs that the kernels see
+    from oracle import transducer_numpy as tn
+
+    tok = x[..., :V].double().numpy()
+    dlp = duration_acts.double().cpu().numpy()
+    denom = tn.denominator(tok)
+    c_ref = np.zeros(B)
+    lg_ref, dg_ref = np.zeros((B, T, U, V)), np.zeros((B, T, U, D))
+    for b in range(B):
+        Tb, Ub = int(al[b]), int(ll[b]) + 1
+        lp = tok[b] + denom[b][..., None]
+        lab_b = [int(v) for v in labels[b][: Ub - 1]]
+        a, llf = tn.tdt_alphas(lp, dlp[b], lab_b, Tb, Ub, V - 1, durations, sigma)
+        bt, _ = tn.tdt_betas(lp, dlp[b], lab_b, Tb, Ub, V - 1, durations, sigma)
+        lg, dg = tn.tdt_grads(lp, dlp[b], a, bt, llf, lab_b, Tb, Ub, V - 1, durations, sigma, lam, clamp)
+        lg_ref[b, :Tb, :Ub], dg_ref[b, :Tb, :Ub] = lg, dg
+        c_ref[b] = -llf * (1.0 + lam)
+    f32 = dtype == torch.float32
+    costs = torch.zeros(B, dtype=dtype, device=DEV)  # rnnt_pytorch.py:145: costs in the dtype of the logits
+    label_grads = torch.full_like(label_acts, float('nan'))
+    duration_grads = torch.full_like(duration_acts, float('nan'))
+    assert rnnt.tdt_loss_gpu(label_acts, duration_acts, lab, ald, lld, costs, label_grads, duration_grads, V - 1,
+                             durations, lam, clamp, 0, sigma, 0.0) is True  # fmt: skip
+    np.testing.assert_allclose(costs.float().cpu().numpy(), c_ref, rtol=1e-5 if f32 else 2.0**-7)
+    tol = 2e-6 if f32 else 2.0**-7
+    assert np.abs(label_grads.float().cpu().numpy() - lg_ref).max() < tol
+    assert np.abs(duration_grads.float().cpu().numpy() - dg_ref).max() < tol
+    # duration_grads is minus an arc posterior: never positive, zero outside the utterance
+    dg = duration_grads.float().cpu().numpy()
+    assert (dg <= 0).all() and (dg[1, al[1]:] == 0).all()
+    # forward only
+    only = torch.zeros(B, dtype=torch.float32, device=DEV)
+    assert rnnt.tdt_loss_gpu(label_acts, duration_acts, lab, ald, lld, only, None, None, V - 1, durations, lam,
+                             clamp, 0, sigma, 0.0) is True  # fmt: skip
+    np.testing.assert_allclose(only.cpu().numpy(), c_ref, rtol=1e-5 if f32 else 2.0**-7)
+    # omega = 1: plain RNNT on the token logits, duration gradient zero (gpu_rnnt.py:606-682)
+    random.seed(3)
+    assert rnnt.tdt_loss_gpu(label_acts, duration_acts, lab, ald, lld, only, label_grads, duration_grads, V - 1,
+                             durations, lam, clamp, 0, sigma, 1.0) is True  # fmt: skip
+    c_r, g_r, _ = oracle.rnnt_loss(x[..., :V].float().numpy(), labels, al, ll, V - 1, lam, clamp)
+    np.testing.assert_allclose(only.cpu().numpy(), c_r, rtol=1e-5)
+    assert np.abs(label_grads.float().cpu().numpy() - g_r).max() < tol
+    assert not duration_grads.any()
+    with pytest.raises(ValueError):
+        rnnt.tdt_loss_gpu(label_acts, duration_acts, lab, ald, lld, only, label_grads, None, V - 1, durations, lam,
+                          clamp, 0, sigma, 0.0)  # fmt: skip
 
 
 def test_timing_hooks_count_the_launches_they_bracket():
