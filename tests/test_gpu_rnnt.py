@@ -319,5 +319,5 @@ def test_vocabularies_just_past_a_power_of_two(V, dtype):
     costs.sum().backward()
     c_ref, g_ref, _ = oracle.rnnt_loss(x.float().numpy(), labels, al, ll, V - 1, 0.01, 0.3)
     f32 = dtype == torch.float32
-    np.testing.assert_allclose(costs.detach().float().cpu().numpy(), c_ref, rtol=1e-6 if f32 else 2.0**-7)
+    np.testing.assert_allclose(costs.detach().float().cpu().numpy(), c_ref, rtol=1e-6 if f32 else 1e-5)
     assert np.abs(acts.grad.float().cpu().numpy() - g_ref).max() < (2e-6 if f32 else 2.0**-8)

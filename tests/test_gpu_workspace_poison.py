@@ -61,9 +61,14 @@ class _PoisonTorch:
 
 
 def _patched(monkeypatch, kind):
-    import speech_amd.joint.fused as fused
-    import speech_amd.k2.rnnt_logprobs as k2
+    import sys
+
+    import speech_amd.joint.fused  # noqa: F401
+    import speech_amd.k2  # noqa: F401
     from speech_amd.rnnt_loss import rnnt, rnnt_pytorch
+
+    # (the package attribute of the same name is the function, hence the look-up by module name)
+    k2, fused = sys.modules["speech_amd.k2.rnnt_logprobs"], sys.modules["speech_amd.joint.fused"]
 
     proxy = _PoisonTorch(kind)
     for mod in (rnnt, rnnt_pytorch, k2, fused):
