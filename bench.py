@@ -9,7 +9,9 @@ lengths), inputs already in HBM.  Prints ONE JSON line:
   roofline     the gradient pass (the dominant kernel; its name for this shape is reported):
                algorithmic bytes per launch / its mean duration, measured with HIP events around
                the launches of the timed steps
-  cpu_baseline the C restatement of the reference's CPU path on a bounded sample, host cores
+  cpu_baseline the C restatement of the reference's CPU path on a bounded sample, host cores (all threads, one
+               thread, and the interpreted per-cell restatement at configuration 1)
+  other_workloads  configurations 3, 4, 5 and the multi-blank one: median ms/step, bytes, fraction of peak
   kernels      mean duration of each pipeline kernel over the timed steps (ms)
   copy_probe   bandwidth a plain device copy reaches on this GPU (GB/s, read + write)
 
@@ -53,49 +55,83 @@ def parse_args():
     ap.add_argument("--op", choices=["loss", "logprobs", "joint"], default="loss")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-graph", action="store_true", help="skip the HIP-graph replay timing of the same step")
+    ap.add_argument("--no-other-workloads", action="store_true",
+                    help="skip the short runs of the other benchmark configurations (default run of workload 1 only)")
     ap.add_argument("--cpu-sample-utterances", type=int, default=16)
     return ap.parse_args()
 
 
 def cpu_baseline(cfg, acts, labels, act_lens, label_lens, n_utt):
     """The reference's CPU path (log_softmax, per-utterance lattice, sparse gradient, softmax
-    Jacobian) restated in C, timed on the host cores over the first n_utt utterances."""
+    Jacobian) restated in C, timed on the host cores over the first n_utt utterances: on all threads (`value`), on one
+    thread over fewer utterances (`c1_value`), and -- for RNNT -- the interpreted per-cell restatement (what a user of
+    the reference gets on a CPU) on the reference's own CPU-sized configuration (`interpreted_cfg1`)."""
     import numpy as np
 
     import oracle
 
     threads = max(1, min(16, os.cpu_count() or 1))
     n_utt = min(n_utt, cfg.B)
-    x = acts[:n_utt].float().cpu().numpy()
-    lab = labels[:n_utt].cpu().numpy()
-    al = act_lens[:n_utt].cpu().numpy()
-    ll = label_lens[:n_utt].cpu().numpy()
     lam, clamp = cfg.fastemit_lambda, max(cfg.clamp, 0.0)
 
-    def one_pass():
-        if cfg.D:
-            oracle.tdt_loss(x, lab, al, ll, cfg.blank, cfg.durations, cfg.sigma, lam, clamp, dtype=np.float32,
-                            num_threads=threads)  # fmt: skip
-        elif cfg.big_blank_durations:
-            oracle.multiblank_loss(x, lab, al, ll, cfg.blank, cfg.big_blank_durations, cfg.sigma, lam, clamp,
-                                   dtype=np.float32, num_threads=threads)  # fmt: skip
-        else:
-            oracle.rnnt_cpu_path(x, lab, al, ll, cfg.blank, lam, clamp, dtype=np.float32, num_threads=threads)
+    def timed(n, nthreads, budget_core_s, max_passes):
+        x = acts[:n].float().cpu().numpy()
+        lab, al, ll = labels[:n].cpu().numpy(), act_lens[:n].cpu().numpy(), label_lens[:n].cpu().numpy()
+
+        def one_pass():
+            if cfg.D:
+                oracle.tdt_loss(x, lab, al, ll, cfg.blank, cfg.durations, cfg.sigma, lam, clamp, dtype=np.float32,
+                                num_threads=nthreads)  # fmt: skip
+            elif cfg.big_blank_durations:
+                oracle.multiblank_loss(x, lab, al, ll, cfg.blank, cfg.big_blank_durations, cfg.sigma, lam, clamp,
+                                       dtype=np.float32, num_threads=nthreads)  # fmt: skip
+            else:
+                oracle.rnnt_cpu_path(x, lab, al, ll, cfg.blank, lam, clamp, dtype=np.float32, num_threads=nthreads)
+
+        passes, t0 = 0, time.perf_counter()
+        while passes < max_passes and (passes == 0 or (time.perf_counter() - t0) * nthreads < budget_core_s):
+            one_pass()
+            passes += 1
+        dt = time.perf_counter() - t0
+        return passes * x.size / dt, passes, dt
 
     # whole passes until about 20 core-seconds of work are spent (at most 8 passes)
-    passes, t0 = 0, time.perf_counter()
-    while passes < 8 and (passes == 0 or (time.perf_counter() - t0) * threads < 20.0):
-        one_pass()
-        passes += 1
-    dt = time.perf_counter() - t0
-    return {
-        "value": passes * x.size / dt,
+    value, passes, dt = timed(n_utt, threads, 20.0, 8)
+    n1 = max(1, min(2, n_utt))
+    c1_value, c1_passes, c1_dt = timed(n1, 1, 5.0, 4)
+    out = {
+        "value": value,
         "unit": "logit elems/s",
         "cores": threads,
         "kind": "port",
         "sample": f"first {n_utt} of {cfg.B} utterances of the same batch, full T x U x V, {passes} pass(es), "
                   f"{dt:.2f} s wall on {threads} threads",
+        "c1_value": c1_value,
+        "c1_sample": f"first {n1} utterance(s), {c1_passes} pass(es), {c1_dt:.2f} s wall on 1 thread",
     }  # fmt: skip
+    if not cfg.D and not cfg.big_blank_durations:
+        out["interpreted_cfg1"] = interpreted_baseline()
+    return out
+
+
+def interpreted_baseline():
+    """The interpreted restatement of the reference's CPU path (per-cell loops over 0-d torch tensors, one thread) on
+    configuration 1 (B=4, T=50, U=21, V=129), checked against the C restatement before its time is reported."""
+    import numpy as np
+
+    import oracle
+    from oracle.cpu_path_interpreted import rnnt_cpu_path_interpreted
+    from speech_amd import synthetic
+
+    cfg1, acts, labels, act_lens, label_lens = synthetic.make_inputs(0)
+    x, lab, al, ll = acts.numpy(), labels.numpy(), act_lens.numpy(), label_lens.numpy()
+    t0 = time.perf_counter()
+    costs, grads = rnnt_cpu_path_interpreted(x, lab, al, ll, cfg1.blank)
+    dt = time.perf_counter() - t0
+    c_ref, g_ref = oracle.rnnt_cpu_path(x, lab, al, ll, cfg1.blank, dtype=np.float64)
+    # the interpreted path keeps its lattice in float32, as the reference does: 5e-4 on the gradient, not 1e-4
+    assert np.allclose(costs, c_ref, rtol=1e-5) and np.abs(grads - g_ref).max() < 5e-4
+    return {"value": x.size / dt, "unit": "logit elems/s", "cores": 1, "workload": cfg1.name, "seconds": dt}
 
 
 def cpu_baseline_logprobs(cfg, acts, labels, act_lens, label_lens, g_target, g_blank, n_utt):
@@ -173,6 +209,56 @@ def graph_replay(torch, cfg, acts, labels, act_lens, label_lens, steps):
     del grads
     return {"ms_per_step": ms, "logit_elems_per_s": cfg.elems / (ms * 1e-3),
             "what": "mi_*_forward + mi_*_backward (grad_output = 1) replayed from one captured HIP graph"}  # fmt: skip
+
+
+def other_workloads(torch, dev, indices, steps=8, warmup=3):
+    """The remaining benchmark configurations, a few steps each, outside the headline's timed region: median step
+    time by stream events, algorithmic bytes and the fraction of the HBM peak of the whole fwd+bwd step."""
+    from speech_amd import MultiblankRNNTLossNumba, RNNTLossNumba, TDTLossNumba, synthetic
+
+    out = []
+    for index in indices:
+        cfg, acts, labels, act_lens, label_lens = synthetic.make_inputs(index, device=dev, generate_on_device=True)
+        acts.requires_grad_(True)
+        if cfg.D:
+            loss = TDTLossNumba(blank=cfg.blank, durations=cfg.durations, reduction='none',
+                                fastemit_lambda=cfg.fastemit_lambda, clamp=cfg.clamp, sigma=cfg.sigma)  # fmt: skip
+        elif cfg.big_blank_durations:
+            loss = MultiblankRNNTLossNumba(blank=cfg.blank, big_blank_durations=cfg.big_blank_durations,
+                                           reduction='none', fastemit_lambda=cfg.fastemit_lambda, clamp=cfg.clamp,
+                                           sigma=cfg.sigma)  # fmt: skip
+        else:
+            loss = RNNTLossNumba(blank=cfg.blank, reduction='none', fastemit_lambda=cfg.fastemit_lambda,
+                                 clamp=cfg.clamp)  # fmt: skip
+        nbytes = synthetic.algorithmic_bytes(cfg, act_lens, label_lens)
+
+        def step():
+            acts.grad = None
+            costs = loss(acts, labels, act_lens, label_lens)
+            costs.sum().backward()
+            return costs
+
+        for _ in range(warmup):
+            step()
+        marks = [torch.cuda.Event(enable_timing=True) for _ in range(steps + 1)]
+        torch.cuda.synchronize()
+        marks[0].record()
+        for i in range(steps):
+            costs = step()
+            marks[i + 1].record()
+        torch.cuda.synchronize()
+        assert bool(torch.isfinite(costs.float()).all()), "non-finite costs"
+        per_step = sorted(marks[i].elapsed_time(marks[i + 1]) for i in range(steps))
+        ms = 0.5 * (per_step[(steps - 1) // 2] + per_step[steps // 2])
+        out.append({
+            "workload": cfg.name, "steps": steps, "ms_per_step": ms, "logit_elems_per_s": cfg.elems / (ms * 1e-3),
+            "algorithmic_bytes": nbytes["total"], "achieved_GBps": nbytes["total"] / (ms * 1e-3) / 1e9,
+            "frac_of_peak": nbytes["total"] / (ms * 1e-3) / 1e9 / HBM_PEAK_GBPS,
+            "dtype": {torch.float32: "f32", torch.bfloat16: "bf16", torch.float16: "f16"}[cfg.dtype],
+        })  # fmt: skip
+        del acts, costs, loss
+        torch.cuda.empty_cache()
+    return out
 
 
 MFMA_BF16_PEAK_TFLOPS = 2500.0  # MI355X dense bf16, published peak
@@ -329,16 +415,18 @@ def main():
     # the timed region: only the dominant kernel is bracketed by events (an event pair costs
     # a few microseconds of queue time; the other kernels are timed in a separate pass below)
     _native.profile_enable(args.steps, ["gradient_pass"])
-    start_ev, stop_ev = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    marks = [torch.cuda.Event(enable_timing=True) for _ in range(args.steps + 1)]
     torch.cuda.synchronize()
     t0 = time.perf_counter()
-    start_ev.record()
-    for _ in range(args.steps):
+    marks[0].record()
+    for i in range(args.steps):
         costs = step()
-    stop_ev.record()
+        marks[i + 1].record()
     torch.cuda.synchronize()
     wall = time.perf_counter() - t0
     kernels = _native.profile_read()
+    per_step = sorted(marks[i].elapsed_time(marks[i + 1]) for i in range(args.steps))
+    median_ms = per_step[len(per_step) // 2] if len(per_step) % 2 else 0.5 * (per_step[len(per_step) // 2 - 1] + per_step[len(per_step) // 2])
     # per-kernel breakdown, outside the timed region
     _native.profile_enable(args.steps)
     for _ in range(args.steps):
@@ -346,8 +434,11 @@ def main():
     torch.cuda.synchronize()
     breakdown = _native.profile_read()
     _native.profile_disable()
-    ms_per_step = wall * 1e3 / args.steps
-    event_ms_per_step = start_ev.elapsed_time(stop_ev) / args.steps
+    # the headline is the MEDIAN step (stream events between the steps of the one timed loop); the mean of the same
+    # loop by the host clock and by the events is reported beside it
+    mean_wall_ms = wall * 1e3 / args.steps
+    event_ms_per_step = marks[0].elapsed_time(marks[-1]) / args.steps
+    ms_per_step = median_ms
     assert bool(torch.isfinite(costs).all()), "non-finite costs"
 
     # copy yardstick: 1 GiB device-to-device
@@ -407,6 +498,10 @@ def main():
             "achieved_GBps": nbytes["total"] / (ms_per_step * 1e-3) / 1e9,
             "frac_of_peak": nbytes["total"] / (ms_per_step * 1e-3) / 1e9 / HBM_PEAK_GBPS,
             "event_ms_per_step": event_ms_per_step,
+            "mean_wall_ms_per_step": mean_wall_ms,
+            "min_ms_per_step": per_step[0],
+            "max_ms_per_step": per_step[-1],
+            "timing": "ms_per_step = median over the timed steps of the stream-event interval of each step",
         },
         "roofline": {
             "kernel": plan["gradient"],
@@ -425,6 +520,11 @@ def main():
         "plan": plan,
         "copy_probe_GBps": copy_gbps,
     }  # fmt: skip
+    if args.workload == 1 and not logprobs and not args.no_other_workloads:
+        del acts, costs
+        torch.cuda.empty_cache()
+        result["other_workloads"] = other_workloads(torch, dev, [2, 3, 4, 5])
+        cfg, acts, labels, act_lens, label_lens = synthetic.make_inputs(1, device=dev, generate_on_device=True)
     if not args.no_graph and not logprobs:
         result["graph_replay"] = graph_replay(torch, cfg, acts.detach(), labels, act_lens, label_lens, args.steps)
     if not args.no_cpu_baseline and logprobs:

@@ -347,7 +347,11 @@ int mi_transducer_export_lattice(const void* workspace, size_t workspace_bytes, 
 int mi_transducer_length_maxima(const int64_t* act_lens, const int64_t* label_lens, int B, int64_t* out,
                                 void* stream);
 
-/* ---- benchmark aids (no counterpart in the reference) --------------------------------
+/* ---- diagnostics ------------------------------------------------------------------------
+ * Everything from here to the end of this header (mi_transducer_profile_*, mi_transducer_describe_plan,
+ * mi_transducer_copy_probe) binds NO interface of the reference: these are aids for benchmarks, profiles and tests
+ * of this library, and a drop-in user of the loss never calls them.
+ *
  * Per-kernel timing of the launches a harness itself makes: after
  * mi_transducer_profile_enable(n, mask), each of the next n launches of every pipeline kernel
  * whose bit (1 << MI_PROFILE_*) is set in mask is bracketed by a pair of HIP events on its
@@ -355,7 +359,9 @@ int mi_transducer_length_maxima(const int64_t* act_lens, const int64_t* label_le
  * costs a few microseconds of queue time, so a harness that also times whole steps should
  * select only the kernel it needs.  mi_transducer_profile_read waits for the recorded
  * launches of one kernel class, returns their summed duration and count, and resets that
- * class.  Not thread-safe; leave disabled outside benchmarks. */
+ * class.  The recording state is the library's only process-wide mutable state; it is guarded by a mutex, so the
+ * calls are safe from any thread, but launches from several threads are then counted into the same classes.  Leave
+ * it disabled outside benchmarks (disabled, a launch only reads one flag). */
 #define MI_PROFILE_DENOM 0   /* denom_rows_kernel / denom_block_kernel / denom_gather_kernel */
 #define MI_PROFILE_LATTICE 1 /* rnnt_lattice_kernel / tdt_lattice_pair_kernel / tdt_lattice_kernel */
 #define MI_PROFILE_CELL 2    /* rnnt_cell_kernel / tdt_cell_kernel */

@@ -15,6 +15,11 @@ INCLUDE_DIR = os.path.join(os.path.dirname(_HERE), "include")
 # MI_TRANSDUCER_LIB lets a kernel developer point at an experimental build of the same ABI
 LIB_PATH = os.environ.get("MI_TRANSDUCER_LIB") or os.path.join(CSRC_DIR, "libmi_transducer.so")
 SOURCES = [os.path.join(CSRC_DIR, "mi_transducer.hip")]
+# the host (CPU) implementation of the RNNT loss: plain C++ / OpenMP, its own library and header
+CPU_LIB_PATH = os.path.join(CSRC_DIR, "libmi_transducer_cpu.so")
+CPU_SOURCES = [os.path.join(CSRC_DIR, "mi_cpu.cpp")]
+CPU_ABI_VERSION = 1
+CXX_FLAGS = ["-O3", "-std=c++17", "-fPIC", "-shared", "-fopenmp", "-Wall", "-Wextra"]
 
 ABI_VERSION = 14
 SUCCESS, INVALID_VALUE, LAUNCH_FAILURE, TOO_LARGE = 0, 1, 2, 3
@@ -32,20 +37,33 @@ HIPCC_FLAGS = [
 ]  # fmt: skip
 
 
-def build(verbose=False):
-    """Compile the HIP sources into speech_amd/csrc/libmi_transducer.so (cross-compiles without a GPU)."""
-    hipcc = os.environ.get("HIPCC", "hipcc")
-    cmd = [hipcc, *HIPCC_FLAGS, "-I", INCLUDE_DIR, "-o", LIB_PATH, *SOURCES]
+def _compile(cmd, what, verbose):
     proc = subprocess.run(cmd, capture_output=True, text=True)
     if verbose or proc.returncode != 0:
         print(" ".join(cmd))
         print(proc.stdout)
         print(proc.stderr)
     if proc.returncode != 0:
-        raise RuntimeError("hipcc failed building libmi_transducer.so:\n" + proc.stderr)
+        raise RuntimeError(f"building {what} failed:\n" + proc.stderr)
+
+
+def build(verbose=False):
+    """Compile the HIP sources into speech_amd/csrc/libmi_transducer.so (cross-compiles without a GPU) and the host
+    implementation of the RNNT loss into speech_amd/csrc/libmi_transducer_cpu.so."""
+    hipcc = os.environ.get("HIPCC", "hipcc")
+    _compile([hipcc, *HIPCC_FLAGS, "-I", INCLUDE_DIR, "-o", LIB_PATH, *SOURCES], "libmi_transducer.so", verbose)
+    build_cpu(verbose)
     global _lib
     _lib = None
     return LIB_PATH
+
+
+def build_cpu(verbose=False):
+    cxx = os.environ.get("CXX", "g++")
+    _compile([cxx, *CXX_FLAGS, "-I", INCLUDE_DIR, "-o", CPU_LIB_PATH, *CPU_SOURCES], "libmi_transducer_cpu.so", verbose)
+    global _cpu_lib
+    _cpu_lib = None
+    return CPU_LIB_PATH
 
 
 _lib = None
@@ -151,6 +169,48 @@ def lib():
             raise RuntimeError(f"libmi_transducer.so has ABI version {got}, expected {ABI_VERSION}: rebuild it")
         _lib = handle
     return _lib
+
+
+_cpu_lib = None
+
+_fp, _i64p = _vp, _vp
+_CPU_SIGNATURES = {
+    "mi_transducer_cpu_abi_version": [],
+    "mi_rnnt_cpu_workspace_bytes": [_c_int, _c_int, _c_int, ctypes.POINTER(_c_size_t)],
+    "mi_rnnt_cpu_forward": [_fp, _i64p, _i64p, _i64p, _fp, _c_int, _c_int, _c_int, _c_int, _c_int, _c_float, _vp,
+                            _c_size_t, _c_int],
+    "mi_rnnt_cpu_backward": [_fp, _i64p, _i64p, _i64p, _fp, _fp, _c_int, _c_float, _c_int, _c_int, _c_int, _c_int,
+                             _c_int, _c_float, _c_float, _c_int, _vp, _c_size_t, _c_int],
+}  # fmt: skip
+CPU_EXPORTED_SYMBOLS = tuple(_CPU_SIGNATURES)
+
+
+def cpu_lib():
+    """The loaded host library; raises if it is missing (there is no other CPU implementation to fall back to)."""
+    global _cpu_lib
+    if _cpu_lib is None:
+        if not os.path.exists(CPU_LIB_PATH):
+            raise RuntimeError(
+                f"{CPU_LIB_PATH} is missing: the host library has not been built "
+                "(run `python -c 'import __graft_entry__ as g; g.build()'`); there is no fallback path"
+            )
+        handle = ctypes.CDLL(CPU_LIB_PATH)
+        for name, argtypes in _CPU_SIGNATURES.items():
+            fn = getattr(handle, name)
+            fn.argtypes = argtypes
+            fn.restype = _c_int
+        got = handle.mi_transducer_cpu_abi_version()
+        if got != CPU_ABI_VERSION:
+            raise RuntimeError(f"libmi_transducer_cpu.so has ABI version {got}, expected {CPU_ABI_VERSION}: rebuild it")
+        _cpu_lib = handle
+    return _cpu_lib
+
+
+def cpu_workspace_bytes(B, T, U):
+    out = _c_size_t(0)
+    if cpu_lib().mi_rnnt_cpu_workspace_bytes(B, T, U, ctypes.byref(out)) != SUCCESS:
+        raise RuntimeError("Invalid parameter passed when calculating working space memory")  # rnnt.py:83-85
+    return int(out.value)
 
 
 def check_status(status, what):

@@ -24,7 +24,9 @@
 #include <math.h>
 #include <stdio.h>
 #include <stdint.h>
+#include <stdlib.h>
 
+#include <atomic>
 #include <mutex>
 #include <type_traits>
 #include <vector>
@@ -44,6 +46,7 @@
 
 namespace {
 
+#include "mi_plan.h"
 #include "mi_device.inc"
 #include "mi_lattice.inc"
 #include "mi_logprobs.inc"
@@ -433,6 +436,8 @@ int mi_transducer_zero_padding(void* grads, int act_dtype, const int64_t* act_le
 
 int mi_transducer_profile_enable(int max_launches, unsigned kernel_mask) {
   if (max_launches <= 0 || max_launches > 65536 || kernel_mask == 0) return MI_TRANSDUCER_INVALID_VALUE;
+  std::lock_guard<std::mutex> lock(g_prof_mutex);
+  g_prof_armed = false;
   g_prof.on = false;
   for (int k = 0; k < MI_PROFILE_KERNELS; ++k) {
     while ((int)g_prof.start[k].size() < max_launches) {
@@ -446,11 +451,13 @@ int mi_transducer_profile_enable(int max_launches, unsigned kernel_mask) {
   g_prof.cap = max_launches;
   g_prof.mask = kernel_mask;
   g_prof.on = true;
+  g_prof_armed = true;
   return MI_TRANSDUCER_SUCCESS;
 }
 
 int mi_transducer_profile_read(int kernel_id, float* total_ms, int* launches) {
   if (kernel_id < 0 || kernel_id >= MI_PROFILE_KERNELS || !total_ms || !launches) return MI_TRANSDUCER_INVALID_VALUE;
+  std::lock_guard<std::mutex> lock(g_prof_mutex);
   float total = 0.f;
   const int n = g_prof.count[kernel_id];
   for (int i = 0; i < n; ++i) {
@@ -467,6 +474,8 @@ int mi_transducer_profile_read(int kernel_id, float* total_ms, int* launches) {
 }
 
 int mi_transducer_profile_disable(void) {
+  std::lock_guard<std::mutex> lock(g_prof_mutex);
+  g_prof_armed = false;
   g_prof.on = false;
   return MI_TRANSDUCER_SUCCESS;
 }

@@ -69,13 +69,25 @@ RNNT_LOSS_RESOLVER = {
 RNNT_LOSS_RESOLVER['default'] = RNNT_LOSS_RESOLVER['warprnnt_numba']
 
 
-def _warn_unused_additional_kwargs(loss_name, kwargs):
-    if len(kwargs) > 0:
-        logging.warning(
-            f"Loss function `{loss_name}` was provided with following additional kwargs,\n"
-            f"however they were ignored as it is unused.\n"
-            f"{kwargs}"
-        )
+def _listed(value, empty):
+    return list(value) if value is not None else empty
+
+
+# name -> (module class, keyword defaults in the order the reference pops them (losses/rnnt.py:264-310), and what
+# to do with a value on its way into the constructor).  Keyword names and defaults are the reference's contract.
+_CONSTRUCTORS = {
+    'warprnnt_numba': (RNNTLossNumba, {'fastemit_lambda': 0.0, 'clamp': -1.0}, {}),
+    'multiblank_rnnt': (
+        MultiblankRNNTLossNumba,
+        {'fastemit_lambda': 0.0, 'clamp': -1.0, 'big_blank_durations': None, 'sigma': 0.0},
+        {'big_blank_durations': lambda v: _listed(v, [])},
+    ),
+    'tdt': (
+        TDTLossNumba,
+        {'fastemit_lambda': 0.0, 'clamp': -1.0, 'durations': None, 'sigma': 0.0, 'omega': 0.0},
+        {'durations': lambda v: _listed(v, None)},
+    ),
+}
 
 
 def resolve_rnnt_default_loss_name() -> str:
@@ -104,44 +116,31 @@ def resolve_rnnt_loss(loss_name: str, blank_idx: int, loss_kwargs: dict = None) 
     if loss_name == 'default':
         loss_name = loss_config.loss_name
 
-    if loss_name == 'warprnnt_numba':
-        fastemit_lambda = loss_kwargs.pop('fastemit_lambda', 0.0)
-        clamp = loss_kwargs.pop('clamp', -1.0)
-        loss_func = RNNTLossNumba(blank=blank_idx, reduction='none', fastemit_lambda=fastemit_lambda, clamp=clamp)
-    elif loss_name == 'multiblank_rnnt':
-        fastemit_lambda = loss_kwargs.pop('fastemit_lambda', 0.0)
-        clamp = loss_kwargs.pop('clamp', -1.0)
-        big_blank_durations = loss_kwargs.pop('big_blank_durations', None)
-        sigma = loss_kwargs.pop('sigma', 0.0)
-        loss_func = MultiblankRNNTLossNumba(
-            blank=blank_idx,
-            big_blank_durations=list(big_blank_durations) if big_blank_durations is not None else [],
-            reduction='none',
-            fastemit_lambda=fastemit_lambda,
-            clamp=clamp,
-            sigma=sigma,
-        )
-    elif loss_name == 'tdt':
-        fastemit_lambda = loss_kwargs.pop('fastemit_lambda', 0.0)
-        clamp = loss_kwargs.pop('clamp', -1.0)
-        durations = loss_kwargs.pop('durations', None)
-        sigma = loss_kwargs.pop('sigma', 0.0)
-        omega = loss_kwargs.pop('omega', 0.0)
-        loss_func = TDTLossNumba(
-            blank=blank_idx,
-            durations=list(durations) if durations is not None else None,
-            reduction='none',
-            fastemit_lambda=fastemit_lambda,
-            clamp=clamp,
-            sigma=sigma,
-            omega=omega,
-        )
-    else:  # an available name without a constructor above: cannot happen while the table and this chain agree
+    if loss_name not in _CONSTRUCTORS:  # an available name without a constructor: the two tables disagree
         raise ValueError(
             f"Invalid value of `loss_name`: {loss_name}. Allowed loss names are :" f"{loss_function_names}"
         )
-    _warn_unused_additional_kwargs(loss_name, loss_kwargs)
+    module_class, defaults, conversions = _CONSTRUCTORS[loss_name]
+    arguments = {key: loss_kwargs.pop(key, default) for key, default in defaults.items()}
+    for key, convert in conversions.items():
+        arguments[key] = convert(arguments[key])
+    loss_func = module_class(blank=blank_idx, reduction='none', **arguments)
+    if loss_kwargs:  # whatever is left was not understood (losses/rnnt.py:161-167)
+        logging.warning(
+            f"Loss function `{loss_name}` was provided with following additional kwargs,\n"
+            f"however they were ignored as it is unused.\n"
+            f"{loss_kwargs}"
+        )
     return loss_func
+
+
+# reduction name -> (per-utterance losses [B], target lengths [B]) -> scalar (losses/rnnt.py:421-436)
+_REDUCTIONS = {
+    'mean_batch': lambda losses, lengths: losses.mean(),
+    'mean': lambda losses, lengths: torch.div(losses, lengths).mean(),
+    'sum': lambda losses, lengths: losses.sum(),
+    'mean_volume': lambda losses, lengths: losses.sum() / lengths.sum(),
+}
 
 
 class RNNTLoss(torch.nn.Module):
@@ -150,7 +149,7 @@ class RNNTLoss(torch.nn.Module):
 
     def __init__(self, num_classes, reduction: str = 'mean_batch', loss_name: str = "default", loss_kwargs=None):
         super().__init__()
-        if reduction not in [None, 'mean', 'sum', 'mean_batch', 'mean_volume']:
+        if reduction is not None and reduction not in _REDUCTIONS:
             raise ValueError('`reduction` must be one of [mean, sum, mean_batch, mean_volume]')
         self._blank = num_classes
         self.reduction = reduction
@@ -158,18 +157,10 @@ class RNNTLoss(torch.nn.Module):
         self._force_float32 = RNNT_LOSS_RESOLVER[loss_name].force_float32
 
     def reduce(self, losses, target_lengths):
-        if isinstance(losses, List):
-            losses = torch.cat(losses, 0)
-            target_lengths = torch.cat(target_lengths, 0)
-        if self.reduction == 'mean_batch':
-            losses = losses.mean()  # global batch size average
-        elif self.reduction == 'mean':
-            losses = torch.div(losses, target_lengths).mean()
-        elif self.reduction == 'sum':
-            losses = losses.sum()
-        elif self.reduction == 'mean_volume':
-            losses = losses.sum() / target_lengths.sum()  # same as above but longer samples weigh more
-        return losses
+        if isinstance(losses, List):  # the fused joint hands over one tensor per sub-batch
+            losses, target_lengths = torch.cat(losses, 0), torch.cat(target_lengths, 0)
+        combine = _REDUCTIONS.get(self.reduction)
+        return losses if combine is None else combine(losses, target_lengths)
 
     def forward(self, *args, log_probs=None, targets=None, input_lengths=None, target_lengths=None):
         if len(args) > 0:  # the reference's @typecheck() (nemo/core/classes/common.py:1357-1359)

@@ -249,6 +249,65 @@ def export_lattice(workspace, act_lens, label_lens, B, T, U, num_durations=0):
     return denom, alphas, betas, llf, llb
 
 
+def _require_cpu_f32(t, what):
+    if t.is_cuda or t.dtype != torch.float32 or not t.is_contiguous():
+        raise ValueError(f"{what} must be a contiguous float32 CPU tensor")
+
+
+def cpu_workspace(acts):
+    B, T, U = acts.shape[:3]
+    return torch.empty(_native.cpu_workspace_bytes(B, T, U) // 8 + 1, dtype=torch.float64)
+
+
+def rnnt_cpu_forward(acts, labels, act_lens, label_lens, costs, blank, fastemit_lambda, workspace, num_threads=0):
+    """costs (float32 [B]) of float32 CPU logits [B,T,U,V]; `workspace` (cpu_workspace) keeps the lattice for
+    rnnt_cpu_backward.  The library applies the log_softmax the reference's module applies with torch."""
+    _require_cpu_f32(acts, "acts")
+    B, T, U, V = acts.shape
+    status = _native.cpu_lib().mi_rnnt_cpu_forward(
+        _ptr(acts), _labels_ptr(labels), _ptr(act_lens), _ptr(label_lens), _ptr(costs), B, T, U, V, int(blank),
+        float(fastemit_lambda), _ptr(workspace), workspace.numel() * 8, int(num_threads),
+    )  # fmt: skip
+    _native.check_status(status, "Could not calculate forward scores")
+
+
+def rnnt_cpu_backward(
+    acts, labels, act_lens, label_lens, grads, grad_scale, blank, fastemit_lambda, clamp, workspace,
+    grad_scale_stride=1, grad_mul=1.0, wrt_log_probs=False, num_threads=0,
+):  # fmt: skip
+    """Gradient w.r.t. the logits (wrt_log_probs: the reference's sparse gradient w.r.t. the log-probs), scaled per
+    utterance by grad_scale[b * stride] * grad_mul and then clamped (clamp > 0)."""
+    _require_cpu_f32(acts, "acts")
+    _require_cpu_f32(grads, "grads")
+    B, T, U, V = acts.shape
+    status = _native.cpu_lib().mi_rnnt_cpu_backward(
+        _ptr(acts), _labels_ptr(labels), _ptr(act_lens), _ptr(label_lens), _ptr(grads), _ptr(grad_scale),
+        int(grad_scale_stride), float(grad_mul), B, T, U, V, int(blank), float(fastemit_lambda), float(clamp),
+        int(bool(wrt_log_probs)), _ptr(workspace), workspace.numel() * 8, int(num_threads),
+    )  # fmt: skip
+    _native.check_status(status, "Could not calculate gradients")
+
+
+def rnnt_loss_cpu(
+    acts, labels, input_lengths, label_lengths, costs, grads, blank_label, fastemit_lambda, clamp, num_threads=0
+):
+    """Drop-in for rnnt.py:39-135: `acts` are LOG-PROBS (the module has applied log_softmax, rnnt_pytorch.py:435);
+    costs (float32 [B]) and grads (or None: forward only) are filled in place, grads with the sparse gradient
+    w.r.t. the log-probs that CPURNNT leaves (cpu_rnnt.py:327-343; `clamp` is not applied here either: the
+    reference clamps in its autograd hook).  num_threads < 0: every core (rnnt.py:83-86)."""
+    del clamp
+    _require_cpu_f32(acts, "acts")
+    if costs.dtype != torch.float32 or costs.is_cuda:
+        raise TypeError("costs must be a float32 CPU tensor")
+    workspace = cpu_workspace(acts)  # raises the reference's RuntimeError for non-positive dims
+    threads = 0 if num_threads < 0 else max(1, int(num_threads))
+    rnnt_cpu_forward(acts, labels, input_lengths, label_lengths, costs, blank_label, fastemit_lambda, workspace, threads)
+    if grads is not None:
+        rnnt_cpu_backward(acts, labels, input_lengths, label_lengths, grads, None, blank_label, fastemit_lambda, 0.0,
+                          workspace, wrt_log_probs=True, num_threads=threads)  # fmt: skip
+    return True
+
+
 def rnnt_loss_gpu(
     acts, labels, input_lengths, label_lengths, costs, grads, blank_label, fastemit_lambda, clamp, num_threads=0
 ):

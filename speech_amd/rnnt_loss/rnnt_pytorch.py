@@ -12,7 +12,8 @@ same outputs: float32 costs of shape [B] (reduction None/'none') or [1]
 
 What is done differently underneath:
   * `acts` are raw logits of dtype float32, bfloat16 or float16 on the GPU; the
-    log-softmax happens inside the kernels.  CPU tensors raise (no CPU path here).
+    log-softmax happens inside the kernels.  CPU tensors go to the host library (RNNT
+    only, as in the reference; TDT and multi-blank raise there as they do in the reference).
   * the gradient is computed in `backward`, by one kernel pass that already folds
     in `grad_output`, the 'mean' reduction's 1/B, FastEmit and the clamp; forward
     keeps a few MB of lattice state instead of a gradient tensor the size of `acts`.
@@ -241,11 +242,23 @@ class _RNNTNumba(Function):
         _certify_static(acts, labels, act_lens, label_lens)
         if clamp < 0:
             raise ValueError("`clamp` must be 0.0 or positive float value.")
-        if not acts.is_cuda:
-            raise RuntimeError(
-                "RNNTLossNumba (MI355X build) has no CPU implementation: move acts, labels and lengths to the GPU"
-            )
         _check_same_device(acts, labels, act_lens, label_lens)
+        ctx.on_cpu = not acts.is_cuda
+        if ctx.on_cpu:
+            # the host library (rnnt_pytorch.py:420-435 + cpu_utils/cpu_rnnt.py): float32 logits in, float32 costs out
+            _PendingLengthCheck(acts, act_lens, label_lens).finish()
+            if acts.dtype != torch.float32:
+                raise TypeError("RNNTLossNumba on CPU tensors computes in float32: the module casts 16-bit logits")
+            need_grad = ctx.needs_input_grad[0]
+            batch = acts.size(0)
+            costs = torch.empty(batch, dtype=torch.float32)
+            workspace = rnnt.cpu_workspace(acts)
+            rnnt.rnnt_cpu_forward(acts, labels, act_lens, label_lens, costs, blank, fastemit_lambda, workspace)
+            costs = _reduce_costs(costs, reduction, batch)
+            if need_grad:
+                ctx.save_for_backward(acts, labels, act_lens, label_lens, workspace)
+                ctx.params = (blank, reduction, fastemit_lambda, clamp)
+            return costs
         pending = _PendingLengthCheck(acts, act_lens, label_lens)
         try:
             need_grad = ctx.needs_input_grad[0]
@@ -276,6 +289,13 @@ class _RNNTNumba(Function):
     def backward(ctx, grad_output):
         acts, labels, act_lens, label_lens, workspace = ctx.saved_tensors
         blank, reduction, fastemit_lambda, clamp = ctx.params
+        if ctx.on_cpu:
+            grads = torch.empty_like(acts)
+            scale, stride, mul = _grad_scale(grad_output, reduction, acts.size(0), acts.device)
+            scale = scale.contiguous()  # (a broadcast grad_output is materialised: B floats)
+            rnnt.rnnt_cpu_backward(acts, labels, act_lens, label_lens, grads, scale, blank, fastemit_lambda, clamp,
+                                   workspace, 1 if scale.numel() > 1 else 0, mul)  # fmt: skip
+            return grads, None, None, None, None, None, None, None
         prepared, ctx.padding = ctx.padding, None  # the prepared buffer serves the first backward call only
         grads = prepared[0] if prepared else grads_like(acts)
         scale, stride, mul = _grad_scale(grad_output, reduction, acts.size(0), acts.device)
@@ -435,6 +455,9 @@ class RNNTLossNumba(Module):
         act_lens: [B] int64 number of valid frames per utterance
         label_lens: [B] int64 number of valid labels per utterance
         """
+        if not acts.is_cuda and acts.dtype != torch.float32:
+            # rnnt_pytorch.py:422-424: 16-bit logits are computed in float32 on the CPU; autograd casts the gradient back
+            acts = acts.float()
         return self.loss(
             acts, labels, act_lens, label_lens, self.blank, self.reduction, self.fastemit_lambda, self.clamp
         )

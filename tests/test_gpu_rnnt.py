@@ -290,8 +290,8 @@ def test_error_behaviour_matches_reference():
     fn.clamp = -0.5
     with pytest.raises(ValueError, match="clamp"):
         fn(acts, lab, al, ll)
-    with pytest.raises(RuntimeError, match="no CPU implementation"):
-        RNNTLossNumba(blank=0)(acts.detach().cpu(), lab.cpu(), al.cpu(), ll.cpu())
+    with pytest.raises(ValueError, match="must be on the device of acts"):
+        RNNTLossNumba(blank=0)(acts.detach(), lab.cpu(), al, ll)
 
 
 def test_loaded_library_is_the_in_tree_build():

@@ -5,6 +5,7 @@ reaches for the oracle."""
 import os
 import re
 
+import numpy as np
 import pytest
 import torch
 
@@ -122,13 +123,28 @@ def test_certify_inputs_on_cpu_tensors():
         certify_inputs(acts, labels, act_lens, label_lens - 1)
 
 
-def test_cpu_tensors_are_refused_loudly():
+def test_cpu_tensors_take_the_host_library_and_tdt_refuses_them():
     acts = torch.zeros(1, 2, 2, 3, requires_grad=True)
     labels = torch.ones(1, 1, dtype=torch.int64)
-    with pytest.raises(RuntimeError, match="no CPU implementation"):
-        RNNTLossNumba()(acts, labels, torch.tensor([2]), torch.tensor([1]))
-    with pytest.raises(ValueError, match="non CUDA"):
+    # all-zero logits, V = 3: every path has probability 3^-(T + U - 1) and there are 2 of them
+    costs = RNNTLossNumba(reduction='none')(acts, labels, torch.tensor([2]), torch.tensor([1]))
+    np.testing.assert_allclose(costs.detach().numpy(), [3 * np.log(3.0) - np.log(2.0)], rtol=1e-6)
+    with pytest.raises(ValueError, match="non CUDA"):  # rnnt_pytorch.py:137-140
         TDTLossNumba(blank=0, durations=[0, 1])(acts, labels, torch.tensor([2]), torch.tensor([1]))
+
+
+def test_host_library_exports_every_symbol_declared_in_its_header():
+    header = open(os.path.join(ROOT, "include", "mi_transducer_cpu.h")).read()
+    declared = set(re.findall(r"^int (mi_[a-z_]+)\(", header, flags=re.M))
+    assert declared == set(_native.CPU_EXPORTED_SYMBOLS)
+    if not os.path.exists(_native.CPU_LIB_PATH):
+        _native.build_cpu()
+    handle = _native.cpu_lib()
+    for name in declared:
+        assert hasattr(handle, name), name
+    assert handle.mi_transducer_cpu_abi_version() == _native.CPU_ABI_VERSION
+    with pytest.raises(RuntimeError):
+        _native.cpu_workspace_bytes(0, 2, 3)
 
 
 def test_missing_library_fails_loudly(monkeypatch, tmp_path):
@@ -141,6 +157,6 @@ def test_missing_library_fails_loudly(monkeypatch, tmp_path):
 def test_package_never_imports_the_oracle():
     for dirpath, _, files in os.walk(os.path.join(ROOT, "speech_amd")):
         for name in files:
-            if name.endswith((".py", ".hip", ".h")):
+            if name.endswith((".py", ".hip", ".h", ".inc", ".cpp")):
                 text = open(os.path.join(dirpath, name)).read()
                 assert "oracle" not in text.lower(), os.path.join(dirpath, name)
