@@ -321,3 +321,29 @@ def test_vocabularies_just_past_a_power_of_two(V, dtype):
     f32 = dtype == torch.float32
     np.testing.assert_allclose(costs.detach().float().cpu().numpy(), c_ref, rtol=1e-6 if f32 else 1e-5)
     assert np.abs(acts.grad.float().cpu().numpy() - g_ref).max() < (2e-6 if f32 else 2.0**-8)
+
+
+def test_length_check_is_memoised_per_tensor_and_version():
+    """The shape-vs-lengths check (rnnt_pytorch.py:628-634) is skipped only for the very tensor objects that
+    already passed it, unmodified; an in-place change or another tensor is checked (and refused) again."""
+    from speech_amd.rnnt_loss import rnnt_pytorch
+
+    rng = np.random.RandomState(3)
+    B, T, U, V = 2, 6, 4, 9
+    acts = torch.tensor(rng.randn(B, T, U, V), dtype=torch.float32, device=DEV)
+    lab, al, ll = to_dev(rng.randint(0, V - 1, size=(B, U - 1)), [T, 4], [U - 1, 2])
+    fn = RNNTLossNumba(blank=V - 1, reduction='none')
+    first = fn(acts, lab, al, ll)
+    entry = rnnt_pytorch._validated.entry
+    assert entry is not None and entry[0]() is al and entry[1]() is ll
+    again = fn(acts, lab, al, ll)  # served from the memo: same result
+    assert torch.equal(first, again)
+    al[0] -= 1  # in place: the version moves, the check runs again and now fails
+    with pytest.raises(ValueError, match="Input length mismatch"):
+        fn(acts, lab, al, ll)
+    al[0] += 1
+    assert torch.equal(fn(acts, lab, al, ll), first)
+    with pytest.raises(ValueError, match="Output length mismatch"):  # another tensor object: always checked
+        fn(acts, lab, al, ll.clone() - 1)
+    with pytest.raises(ValueError, match="Input length mismatch"):  # same tensors against another shape
+        fn(acts[:, : T - 1].contiguous(), lab, al, ll)
