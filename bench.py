@@ -57,6 +57,9 @@ def parse_args():
     ap.add_argument("--no-graph", action="store_true", help="skip the HIP-graph replay timing of the same step")
     ap.add_argument("--no-other-workloads", action="store_true",
                     help="skip the short runs of the other benchmark configurations (default run of workload 1 only)")
+    ap.add_argument("--lattice", choices=["auto", "log", "scaled"], default="auto",
+                    help="lattice kernels: auto = the library's default per loss, log = always the log-domain "
+                         "recursions, scaled = the probability-domain recursions wherever the shape allows (A/B timing)")
     ap.add_argument("--cpu-sample-utterances", type=int, default=16)
     return ap.parse_args()
 
@@ -365,6 +368,7 @@ def main():
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
     _native.lib()  # fail now if the HIP library is missing
+    _native.check_status(_native.lib().mi_transducer_set_lattice_mode({"auto": 0, "log": 1, "scaled": 2}[args.lattice]), "lattice mode")
 
     cfg, acts, labels, act_lens, label_lens = synthetic.make_inputs(args.workload, device=dev, generate_on_device=True)
     if args.op == "joint":

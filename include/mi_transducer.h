@@ -349,7 +349,7 @@ int mi_transducer_length_maxima(const int64_t* act_lens, const int64_t* label_le
 
 /* ---- diagnostics ------------------------------------------------------------------------
  * Everything from here to the end of this header (mi_transducer_profile_*, mi_transducer_describe_plan,
- * mi_transducer_copy_probe) binds NO interface of the reference: these are aids for benchmarks, profiles and tests
+ * mi_transducer_copy_probe, mi_transducer_set_lattice_mode, mi_transducer_scale_segment) binds NO interface of the reference: these are aids for benchmarks, profiles and tests
  * of this library, and a drop-in user of the loss never calls them.
  *
  * Per-kernel timing of the launches a harness itself makes: after
@@ -363,7 +363,7 @@ int mi_transducer_length_maxima(const int64_t* act_lens, const int64_t* label_le
  * calls are safe from any thread, but launches from several threads are then counted into the same classes.  Leave
  * it disabled outside benchmarks (disabled, a launch only reads one flag). */
 #define MI_PROFILE_DENOM 0   /* denom_rows_kernel / denom_block_kernel / denom_gather_kernel */
-#define MI_PROFILE_LATTICE 1 /* rnnt_lattice_kernel / tdt_lattice_pair_kernel / tdt_lattice_kernel */
+#define MI_PROFILE_LATTICE 1 /* rnnt_scaled_lattice_kernel / rnnt_lattice_kernel / tdt_lattice_pair_kernel / tdt_lattice_kernel */
 #define MI_PROFILE_CELL 2    /* rnnt_cell_kernel / tdt_cell_kernel */
 #define MI_PROFILE_GRAD 3    /* grad_rows_kernel / grad_block_kernel / grad_stream_kernel */
 #define MI_PROFILE_ZERO 4    /* zero_padding_kernel */
@@ -385,6 +385,19 @@ int mi_transducer_describe_plan(int act_dtype, int B, int T, int U, int V, int D
  * one-vector-per-thread kernel (the fastest streaming pattern measured): the known-size yardstick for hardware traffic
  * counters and for the copy bandwidth the GPU reaches in practice. */
 int mi_transducer_copy_probe(const void* src, void* dst, size_t bytes, void* stream);
+
+/* Which lattice kernels the forward calls run (process-wide): 0 (the default) = per loss, whichever measured
+ * faster; 1 = always the log-domain recursions; 2 = the scaled, probability-domain recursions wherever the shape
+ * allows them (each returns to the log domain per utterance when its own checks ask for it).  For tests that hold
+ * one against the other and for A/B timing. */
+int mi_transducer_set_lattice_mode(int mode);
+
+/* Where a workspace of this shape keeps, per utterance, the word that says which format the last RNNT lattice
+ * kernel left alphas and betas in (0 = natural logs, 1 = scaled probabilities): int32 number
+ * `*format_word` of the `*ints_per_utterance` ints that start at byte `*offset_bytes + 4 * b * *ints_per_utterance`.
+ * Host arithmetic only.  For tests that must know which of the two recursions produced a result. */
+int mi_transducer_scale_segment(int B, int T, int U, int D, size_t* offset_bytes, int* ints_per_utterance,
+                                int* format_word);
 
 #ifdef __cplusplus
 }

@@ -21,7 +21,7 @@ CPU_SOURCES = [os.path.join(CSRC_DIR, "mi_cpu.cpp")]
 CPU_ABI_VERSION = 1
 CXX_FLAGS = ["-O3", "-std=c++17", "-fPIC", "-shared", "-fopenmp", "-Wall", "-Wextra"]
 
-ABI_VERSION = 14
+ABI_VERSION = 15
 SUCCESS, INVALID_VALUE, LAUNCH_FAILURE, TOO_LARGE = 0, 1, 2, 3
 STATIC_WORKSPACE_BYTES = 64 << 20
 DTYPE_F32, DTYPE_BF16, DTYPE_F16 = 0, 1, 2
@@ -145,6 +145,8 @@ _SIGNATURES = {
     "mi_transducer_describe_plan": [_c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int,
                                     ctypes.c_char_p, _c_size_t],
     "mi_transducer_copy_probe": [_vp, _vp, _c_size_t, _vp],
+    "mi_transducer_set_lattice_mode": [_c_int],
+    "mi_transducer_scale_segment": [_c_int, _c_int, _c_int, _c_int, _vp, _vp, _vp],
 }  # fmt: skip
 
 EXPORTED_SYMBOLS = tuple(_SIGNATURES)

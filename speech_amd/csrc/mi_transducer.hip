@@ -64,7 +64,7 @@ namespace {
 // ----------------------------------------------------------------------------------------
 extern "C" {
 
-int mi_transducer_abi_version(void) { return 14; }
+int mi_transducer_abi_version(void) { return 15; }
 
 int mi_transducer_workspace_bytes(int B, int T, int U, int D, size_t* out_bytes) {
   Layout L;
@@ -81,8 +81,9 @@ int mi_rnnt_forward(const void* acts, int act_dtype, const int64_t* labels, cons
   int st = check_common(acts, act_dtype, labels, act_lens, label_lens, B, T, U, V, 0, blank, workspace,
                         workspace_bytes, stream, &c);
   if (st) return st;
-  if ((st = run_denom(c))) return st;
-  return run_rnnt_lattice(c, costs, fastemit_lambda, with_betas);
+  const unsigned long long mark = scaled_lattice_mark(c, with_betas);
+  if ((st = run_denom(c, mark))) return st;
+  return run_rnnt_lattice(c, costs, fastemit_lambda, with_betas, mark);
 }
 
 int mi_rnnt_backward(const void* acts, int act_dtype, const int64_t* labels, const int64_t* act_lens,
@@ -363,9 +364,27 @@ int mi_transducer_export_lattice(const void* workspace, size_t workspace_bytes, 
   const unsigned grid = (unsigned)((cells + 255) / 256);
   hipLaunchKernelGGL(export_lattice_kernel, dim3(grid), dim3(256), 0, (hipStream_t)stream,
                      (const float*)(ws + L.off_denom), (const double*)(ws + L.off_alphas),
-                     (const double*)(ws + L.off_betas), (const double*)(ws + L.off_ll), act_lens, label_lens, denom,
-                     alphas, betas, ll_forward, ll_backward, B, T, U, L.ND, L.Us, cells);
+                     (const double*)(ws + L.off_betas), (const double*)(ws + L.off_ll),
+                     D == 0 ? (const int*)(ws + L.off_scale) : nullptr, L.SG, act_lens, label_lens, denom, alphas, betas,
+                     ll_forward, ll_backward, B, T, U, L.ND, L.Us, cells);
   return launch_status();
+}
+
+int mi_transducer_scale_segment(int B, int T, int U, int D, size_t* offset_bytes, int* ints_per_utterance,
+                                int* format_word) {
+  Layout L;
+  if (!offset_bytes || !ints_per_utterance || !format_word || !make_layout(B, T, U, D, &L))
+    return MI_TRANSDUCER_INVALID_VALUE;
+  *offset_bytes = L.off_scale;
+  *ints_per_utterance = L.SG;
+  *format_word = kScaleFormat;
+  return MI_TRANSDUCER_SUCCESS;
+}
+
+int mi_transducer_set_lattice_mode(int mode) {
+  if (mode < 0 || mode > 2) return MI_TRANSDUCER_INVALID_VALUE;
+  g_lattice_mode.store(mode, std::memory_order_relaxed);
+  return MI_TRANSDUCER_SUCCESS;
 }
 
 int mi_transducer_length_maxima(const int64_t* act_lens, const int64_t* label_lens, int B, int64_t* out,

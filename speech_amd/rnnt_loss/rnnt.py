@@ -249,6 +249,34 @@ def export_lattice(workspace, act_lens, label_lens, B, T, U, num_durations=0):
     return denom, alphas, betas, llf, llb
 
 
+def set_lattice_mode(mode):
+    """0: per loss, whichever lattice kernel measured faster; 1: always the log-domain recursions; 2: the scaled
+    (probability-domain) recursions wherever the shape allows them.  Process-wide; for tests and A/B timing."""
+    _native.check_status(_native.lib().mi_transducer_set_lattice_mode(int(mode)), "set_lattice_mode")
+
+
+def lattice_formats(workspace, B, T, U, num_durations=0):
+    """int32[B]: per utterance, the format the last RNNT lattice kernel left in `workspace` (0 logs, 1 scaled)."""
+    off, per, word = ctypes.c_size_t(0), ctypes.c_int(0), ctypes.c_int(0)
+    status = _native.lib().mi_transducer_scale_segment(
+        B, T, U, num_durations, ctypes.byref(off), ctypes.byref(per), ctypes.byref(word)
+    )
+    _native.check_status(status, "scale_segment")
+    seg = workspace[off.value : off.value + 4 * per.value * B].view(torch.int32).view(B, per.value)
+    return seg[:, word.value].clone()
+
+
+def lattice_diagnostics(workspace, B, T, U):
+    """int32[B, 2] of the scaled RNNT lattice kernel: why an utterance took the log route (bit 0 an arc probability
+    out of range, bits 1 / 2 a direction ran out of range, bit 3 the exponent bound, bit 4 totals differ; 0 if it
+    did not), and the exponent spread it measured."""
+    off, per, word = ctypes.c_size_t(0), ctypes.c_int(0), ctypes.c_int(0)
+    status = _native.lib().mi_transducer_scale_segment(B, T, U, 0, ctypes.byref(off), ctypes.byref(per), ctypes.byref(word))
+    _native.check_status(status, "scale_segment")
+    seg = workspace[off.value : off.value + 4 * per.value * B].view(torch.int32).view(B, per.value)
+    return seg[:, 2:4].clone()
+
+
 def _require_cpu_f32(t, what):
     if t.is_cuda or t.dtype != torch.float32 or not t.is_contiguous():
         raise ValueError(f"{what} must be a contiguous float32 CPU tensor")
