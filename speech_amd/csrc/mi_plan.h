@@ -35,7 +35,8 @@ struct Layout {
   int A;    // arc planes per diagonal row: blank, label, D duration log-probs
   int CS;   // floats per cell in the coefficient buffer
   int SG;   // ints per utterance in the scale segment: kScaleHeader, then {alpha, beta} exponent per 8 diagonals
-  size_t off_denom, off_arcs, off_alphas, off_betas, off_ll, off_coef, off_arcp, off_scale, total;
+  size_t off_denom, off_arcs, off_alphas, off_betas, off_ll, off_coef, off_scale, total;
+  size_t off_arcp, total_scaled;  // total_scaled = total + the arc-probability segment of the scaled RNNT lattice
 };
 
 inline size_t align256(size_t x) { return (x + 255) & ~(size_t)255; }
@@ -58,13 +59,15 @@ inline bool make_layout(int B, int T, int U, int D, Layout* L) {
   L->off_betas = off;  off = align256(off + skew * sizeof(double));
   L->off_ll = off;     off = align256(off + (size_t)B * 2 * sizeof(double));
   L->off_coef = off;   off = align256(off + cells * L->CS * sizeof(float));
-  // the scaled (probability-domain) RNNT lattice: blank / label arc PROBABILITIES as doubles, skewed like `arcs`
-  // (plain RNNT only), and per utterance a header (which format the lattice is in, the total probability) followed
-  // by the binary exponents of the alpha and beta values of every block of kScaleBlock anti-diagonals
+  // per utterance a header (which format the lattice is in, the total probability) followed by the binary exponents
+  // of the alpha and beta values of every block of kScaleBlock anti-diagonals of a scaled lattice
   L->SG = kScaleHeader + 2 * ((L->ND / kScaleBlock + 3) & ~1);
-  L->off_arcp = off;   off = align256(off + (D == 0 ? skew * 2 * sizeof(double) : 0));
   L->off_scale = off;  off = align256(off + (size_t)B * L->SG * sizeof(int));
   L->total = off;
+  // the scaled (probability-domain) RNNT lattice also wants the blank / label arc PROBABILITIES as doubles, skewed
+  // like `arcs`: a segment behind everything else that only a caller who asked for that lattice has to bring
+  L->off_arcp = off;   off = align256(off + (D == 0 ? skew * 2 * sizeof(double) : 0));
+  L->total_scaled = off;
   return true;
 }
 

@@ -69,7 +69,8 @@ int mi_transducer_abi_version(void) { return 15; }
 int mi_transducer_workspace_bytes(int B, int T, int U, int D, size_t* out_bytes) {
   Layout L;
   if (!out_bytes || !make_layout(B, T, U, D, &L)) return MI_TRANSDUCER_INVALID_VALUE;
-  *out_bytes = L.total;
+  // (the scaled RNNT lattice, lattice mode 2, keeps one more segment)
+  *out_bytes = g_lattice_mode.load(std::memory_order_relaxed) == 2 ? L.total_scaled : L.total;
   return MI_TRANSDUCER_SUCCESS;
 }
 
@@ -412,7 +413,7 @@ int mi_rnnt_lattice(const int64_t* act_lens, const int64_t* label_lens, float* c
     return MI_TRANSDUCER_INVALID_VALUE;
   c.act_lens = act_lens; c.label_lens = label_lens;
   c.B = B; c.T = T; c.U = U; c.D = D;
-  c.ws = (char*)workspace; c.stream = (hipStream_t)stream;
+  c.ws = (char*)workspace; c.ws_bytes = workspace_bytes; c.stream = (hipStream_t)stream;
   return run_rnnt_lattice(c, costs, fastemit_lambda, with_betas);
 }
 
@@ -428,7 +429,7 @@ int mi_tdt_lattice(const int64_t* act_lens, const int64_t* label_lens, float* co
     return MI_TRANSDUCER_INVALID_VALUE;
   c.act_lens = act_lens; c.label_lens = label_lens;
   c.B = B; c.T = T; c.U = U; c.D = D;
-  c.ws = (char*)workspace; c.stream = (hipStream_t)stream;
+  c.ws = (char*)workspace; c.ws_bytes = workspace_bytes; c.stream = (hipStream_t)stream;
   return run_tdt_lattice(c, costs, fastemit_lambda, with_betas, prm);
 }
 
