@@ -243,10 +243,12 @@ int mi_rnnt_logprobs_backward(const void* logits, int act_dtype, const int64_t* 
 /* ---- joint projection fused into the forward pass --------------------------------------
  * Replaces RNNTJoint.joint_after_projection followed by the loss forward
  * (nemo/collections/asr/modules/rnnt.py:1707-1724 and :1573-1578) for the default joint network
- * (ReLU, optional Dropout, Linear(H -> V); :1759-1777): the [B,T,U,V] tensor is never written.
+ * (activation, optional Dropout, Linear(H -> V); :1759-1777): the [B,T,U,V] tensor is never written.
+ * `activation`: 0 ReLU, 1 tanh, 2 sigmoid (the three the reference accepts, :1762-1770); the activation's output is
+ * rounded to bf16 as torch's is, and the backward takes its slope at that rounded output.
  *   f [B,T,H], g [B,U,H]: bf16, the projected encoder / prediction-network outputs (16-byte aligned);
  *   weight [V,H], bias [V] (nullable): float32 or bf16 (weight_dtype), the final Linear layer;
- *   logits = relu(f[b,t] + g[b,u]) . weight^T + bias with bf16 operands and float32 accumulation
+ *   logits = act(f[b,t] + g[b,u]) . weight^T + bias with bf16 operands and float32 accumulation
  *   (what the reference computes under bf16 autocast, minus its rounding of the logits to bf16).
  * costs[b] as mi_rnnt_forward; the workspace (mi_joint_workspace_bytes) ends up holding the same
  * lattice state.  H must be one of 256, 320, 384, 512, 640; V any.
@@ -264,17 +266,17 @@ int mi_rnnt_logprobs_backward(const void* logits, int act_dtype, const int64_t* 
 int mi_joint_workspace_bytes(int B, int T, int U, int H, int V, int D, int num_big_blanks, size_t* out_bytes);
 int mi_joint_rnnt_forward(const void* f, const void* g, const void* weight, const void* bias, int weight_dtype,
                           const int64_t* labels, const int64_t* act_lens, const int64_t* label_lens, float* costs,
-                          int* tile_count, float dropout_p, unsigned long long dropout_seed, int B, int T, int U, int H,
+                          int* tile_count, float dropout_p, unsigned long long dropout_seed, int activation, int B, int T, int U, int H,
                           int V, int blank, float fastemit_lambda, int with_betas, void* workspace,
                           size_t workspace_bytes, void* stream);
 int mi_joint_tdt_forward(const void* f, const void* g, const void* weight, const void* bias, int weight_dtype,
                          const int64_t* labels, const int64_t* act_lens, const int64_t* label_lens, float* costs,
-                         int* tile_count, float dropout_p, unsigned long long dropout_seed, int B, int T, int U, int H,
+                         int* tile_count, float dropout_p, unsigned long long dropout_seed, int activation, int B, int T, int U, int H,
                          int V, int D, const int32_t* durations_host, int blank, float fastemit_lambda, float sigma,
                          int with_betas, void* workspace, size_t workspace_bytes, void* stream);
 int mi_joint_multiblank_forward(const void* f, const void* g, const void* weight, const void* bias, int weight_dtype,
                                 const int64_t* labels, const int64_t* act_lens, const int64_t* label_lens, float* costs,
-                                int* tile_count, float dropout_p, unsigned long long dropout_seed, int B, int T, int U,
+                                int* tile_count, float dropout_p, unsigned long long dropout_seed, int activation, int B, int T, int U,
                                 int H, int V, int num_big_blanks, const int32_t* big_blank_durations_host, int blank,
                                 float fastemit_lambda, float sigma, int with_betas, void* workspace,
                                 size_t workspace_bytes, void* stream);
@@ -298,31 +300,31 @@ int mi_joint_padded_vocabulary(int V);
 int mi_joint_rnnt_backward_logits(const void* f, const void* g, const int64_t* labels, const int64_t* act_lens,
                                   const int64_t* label_lens, void* dlogits, void* hidden, int tiles,
                                   const float* grad_scale, int grad_scale_stride,
-                                  float grad_mul, float dropout_p, unsigned long long dropout_seed, int B, int T, int U,
+                                  float grad_mul, float dropout_p, unsigned long long dropout_seed, int activation, int B, int T, int U,
                                   int H, int V, int blank, float fastemit_lambda, float clamp, void* workspace,
                                   size_t workspace_bytes, void* stream);
 int mi_joint_tdt_backward_logits(const void* f, const void* g, const int64_t* labels, const int64_t* act_lens,
                                  const int64_t* label_lens, void* dlogits, void* hidden, int tiles,
                                  const float* grad_scale, int grad_scale_stride, float grad_mul, float dropout_p,
-                                 unsigned long long dropout_seed, int B, int T, int U, int H, int V, int D,
+                                 unsigned long long dropout_seed, int activation, int B, int T, int U, int H, int V, int D,
                                  const int32_t* durations_host, int blank, float fastemit_lambda, float clamp,
                                  float sigma, void* workspace, size_t workspace_bytes, void* stream);
 int mi_joint_multiblank_backward_logits(const void* f, const void* g, const int64_t* labels, const int64_t* act_lens,
                                         const int64_t* label_lens, void* dlogits, void* hidden, int tiles,
                                         const float* grad_scale, int grad_scale_stride, float grad_mul,
-                                        float dropout_p, unsigned long long dropout_seed, int B, int T, int U, int H,
+                                        float dropout_p, unsigned long long dropout_seed, int activation, int B, int T, int U, int H,
                                         int V, int num_big_blanks, const int32_t* big_blank_durations_host, int blank,
                                         float fastemit_lambda, float clamp, float sigma, void* workspace,
                                         size_t workspace_bytes, void* stream);
 
 /* Backward of the fused joint, last step: d_hidden [rows][H] bf16 (= dlogits . weight, rows as above) times the
- * ReLU derivative, summed over u into d_f [B,T,H] and over t into d_g [B,U,H] (float32; either may be NULL; frames
+ * activation's derivative, summed over u into d_f [B,T,H] and over t into d_g [B,U,H] (float32; either may be NULL; frames
  * and label positions outside an utterance get zeros).  The derivative is recomputed from f and g (the forward
  * call's bf16 inputs), `tiles` is the same count as in mi_joint_rnnt_backward_logits, the workspace the forward
  * call's. */
 int mi_joint_reduce_hidden(const void* d_hidden, const void* f, const void* g, const int64_t* act_lens,
                            const int64_t* label_lens, float* d_f, float* d_g, int tiles, float dropout_p,
-                           unsigned long long dropout_seed, int B, int T, int U, int H, int V, int D,
+                           unsigned long long dropout_seed, int activation, int B, int T, int U, int H, int V, int D,
                            int num_big_blanks, void* workspace, size_t workspace_bytes, void* stream);
 
 /* Where the forward call left the packed weights inside its workspace: *rows x *pitch bf16, row n = weight[n, :]

@@ -195,11 +195,12 @@ def rnnt_logprobs_grad(logits, targets, blank, grad_target_scores, grad_blank_sc
 
 
 def joint_rnnt_loss(f, g, weight, bias, labels, act_lens, label_lens, blank, fastemit_lambda=0.0, clamp=0.0, grad_costs=None,
-                    keep_mask=None, dropout_p=0.0, durations=None, sigma=0.0, big_blank_durations=None):
+                    keep_mask=None, dropout_p=0.0, durations=None, sigma=0.0, big_blank_durations=None,
+                    activation="relu"):
     """Joint network + RNNT / TDT / multi-blank loss (numpy restatement; see transducer_numpy.joint_rnnt_loss)."""
     from oracle import transducer_numpy
 
     return transducer_numpy.joint_rnnt_loss(
         f, g, weight, bias, labels, act_lens, label_lens, blank, fastemit_lambda, clamp, grad_costs, keep_mask, dropout_p,
-        durations, sigma, big_blank_durations,
+        durations, sigma, big_blank_durations, activation,
     )

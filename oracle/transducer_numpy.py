@@ -652,9 +652,12 @@ def bf16_round(x):
 
 
 def joint_rnnt_loss(f, g, weight, bias, labels, act_lens, label_lens, blank, fastemit_lambda=0.0, clamp=0.0, grad_costs=None,
-                    keep_mask=None, dropout_p=0.0, durations=None, sigma=0.0, big_blank_durations=None):
-    """RNNT (with `durations` TDT, with `big_blank_durations` multi-blank) loss of the ReLU joint's logits under
-    bf16-autocast arithmetic, and its gradients.
+                    keep_mask=None, dropout_p=0.0, durations=None, sigma=0.0, big_blank_durations=None,
+                    activation="relu"):
+    """RNNT (with `durations` TDT, with `big_blank_durations` multi-blank) loss of the joint's logits under
+    bf16-autocast arithmetic, and its gradients.  `activation`: relu, tanh or sigmoid (modules/rnnt.py:1762-1770);
+    where "relu" stands below read act(x) rounded to bf16, with the derivative taken at that rounded output
+    (1 - h^2, h (1 - h)) as torch's tanh / sigmoid backward does.
 
     logits[b,t,u,:] = drop(relu(bf16(f[b,t] + g[b,u]))) @ bf16(weight).T + bias   (modules/rnnt.py:1707-1724,
     joint_net = ReLU, Dropout, Linear :1766-1777; operands rounded to bf16, products and sums exact here --
@@ -678,8 +681,17 @@ def joint_rnnt_loss(f, g, weight, bias, labels, act_lens, label_lens, blank, fas
         b_hi = bf16_round(bias)
         b_eff = b_hi + bf16_round(np.asarray(bias, dtype=np.float32) - b_hi.astype(np.float32))
     pre = bf16_round(f[:, :, None, :] + g[:, None, :, :])  # [B,T,U,H]
-    hidden = np.maximum(pre, 0.0)
-    chain = (pre > 0).astype(np.float64)  # d hidden / d pre
+    if activation == "relu":
+        hidden = np.maximum(pre, 0.0)
+        chain = (pre > 0).astype(np.float64)  # d hidden / d pre
+    elif activation == "tanh":
+        hidden = bf16_round(np.tanh(pre))
+        chain = 1.0 - hidden * hidden
+    elif activation == "sigmoid":
+        hidden = bf16_round(1.0 / (1.0 + np.exp(-pre)))
+        chain = hidden * (1.0 - hidden)
+    else:
+        raise ValueError(activation)
     if keep_mask is not None:
         scale = np.float32(1.0) / (np.float32(1.0) - np.float32(dropout_p))
         keep = np.asarray(keep_mask, dtype=bool)

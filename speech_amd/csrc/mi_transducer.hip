@@ -64,7 +64,7 @@ namespace {
 // ----------------------------------------------------------------------------------------
 extern "C" {
 
-int mi_transducer_abi_version(void) { return 15; }
+int mi_transducer_abi_version(void) { return 16; }
 
 int mi_transducer_workspace_bytes(int B, int T, int U, int D, size_t* out_bytes) {
   Layout L;

@@ -227,22 +227,48 @@ def multiblank_autograd(logits, labels, blank, big_blank_durations, sigma, lam=0
     return float(nll.detach()) * (1.0 + lam), x.grad.numpy()
 
 
-def joint_autograd(f, g, weight, bias, labels, blank, grad_costs, keep_mask=None, dropout_p=0.0):
-    """Costs and gradients of sum_b grad_costs[b] * nll_b through relu(f+g) @ W.T + bias, all utterances at
+class _RoundedActivation(torch.autograd.Function):
+    """tanh / sigmoid whose output is rounded to bf16 and whose backward takes the slope at that rounded output
+    (torch's tanh_backward / sigmoid_backward get the OUTPUT tensor, which under autocast is the bf16 one)."""
+
+    @staticmethod
+    def forward(ctx, x, kind):
+        out = (torch.tanh(x) if kind == "tanh" else torch.sigmoid(x)).float().to(torch.bfloat16).double()
+        ctx.save_for_backward(out)
+        ctx.kind = kind
+        return out
+
+    @staticmethod
+    def backward(ctx, grad):
+        (out,) = ctx.saved_tensors
+        return grad * ((1.0 - out * out) if ctx.kind == "tanh" else out * (1.0 - out)), None
+
+
+def joint_autograd(f, g, weight, bias, labels, blank, grad_costs, keep_mask=None, dropout_p=0.0, activation="relu",
+                   rounded_activation=True):
+    """Costs and gradients of sum_b grad_costs[b] * nll_b through act(f+g) @ W.T + bias, all utterances at
     full length, by torch autograd in float64; `f`, `g`, `weight`, `bias` must already be exactly
-    representable in bf16, and the rounding of f+g to bf16 is applied straight-through."""
+    representable in bf16, and the rounding of f+g to bf16 is applied straight-through.  tanh / sigmoid outputs are
+    rounded to bf16 with the slope taken there (rounded_activation=False: plain float64 tanh / sigmoid, for a
+    loose cross-check that owes nothing to that convention)."""
     f = torch.tensor(np.asarray(f, dtype=np.float64), requires_grad=True)
     g = torch.tensor(np.asarray(g, dtype=np.float64), requires_grad=True)
     w = torch.tensor(np.asarray(weight, dtype=np.float64), requires_grad=True)
     b = torch.tensor(np.asarray(bias, dtype=np.float64), requires_grad=True)
     s = f[:, :, None, :] + g[:, None, :, :]
     s = s + (s.detach().float().to(torch.bfloat16).double() - s.detach())
-    hidden = torch.relu(s)
+    if activation == "relu":
+        hidden = torch.relu(s)
+    elif rounded_activation:
+        hidden = _RoundedActivation.apply(s, activation)
+    else:
+        hidden = torch.tanh(s) if activation == "tanh" else torch.sigmoid(s)
+    act_out = hidden
     if keep_mask is not None:  # dropout with a given mask; its bf16 output rounding is straight-through as well
         scale = float(np.float32(1.0) / (np.float32(1.0) - np.float32(dropout_p)))
         hidden = hidden * torch.tensor(np.asarray(keep_mask, dtype=np.float64)) * scale
         # the product is formed in float32 before the rounding, as on the GPU
-        exact32 = (torch.relu(s).detach().float() * np.float32(scale)).to(torch.bfloat16).double()
+        exact32 = (act_out.detach().float() * np.float32(scale)).to(torch.bfloat16).double()
         rounded = torch.where(torch.tensor(np.asarray(keep_mask, dtype=bool)), exact32, torch.zeros_like(exact32))
         hidden = hidden + (rounded - hidden.detach())
     logits = torch.nn.functional.linear(hidden, w, b)

@@ -38,19 +38,21 @@ def dev_ints(*arrays):
     return [torch.tensor(np.asarray(a), dtype=torch.int64, device=DEV) for a in arrays]
 
 
-def check(seed, B, T, U, H, V, lam=0.0, clamp=0.0, ragged=True, bias_on=True, weight_dtype=torch.float32):
+def check(seed, B, T, U, H, V, lam=0.0, clamp=0.0, ragged=True, bias_on=True, weight_dtype=torch.float32,
+          activation="relu"):
     f, g, W, bias, labels, al, ll = make_case(seed, B, T, U, H, V, ragged)
     rng = np.random.RandomState(seed + 1000)
     gc = (rng.rand(B) + 0.5).astype(np.float32)
     Wq = W.to(weight_dtype)
     bq = bias.to(weight_dtype) if bias_on else None
     ref = oracle.joint_rnnt_loss(f.float().numpy(), g.float().numpy(), Wq.float().numpy(),
-                                 None if bq is None else bq.float().numpy(), labels, al, ll, V - 1, lam, clamp, gc)  # fmt: skip
+                                 None if bq is None else bq.float().numpy(), labels, al, ll, V - 1, lam, clamp, gc,
+                                 activation=activation)  # fmt: skip
     fd, gd = f.to(DEV).requires_grad_(True), g.to(DEV).requires_grad_(True)
     Wd = Wq.to(DEV).requires_grad_(True)
     bd = None if bq is None else bq.to(DEV).requires_grad_(True)
     lab, ald, lld = dev_ints(labels, al, ll)
-    costs = joint_rnnt_loss(fd, gd, Wd, bd, lab, ald, lld, V - 1, lam, clamp)
+    costs = joint_rnnt_loss(fd, gd, Wd, bd, lab, ald, lld, V - 1, lam, clamp, activation=activation)
     (costs * torch.tensor(gc, device=DEV)).sum().backward()
     torch.cuda.synchronize()
     assert costs.dtype == torch.float32 and costs.shape == (B,)
@@ -72,6 +74,19 @@ def test_small_lattices_every_vocabulary_tiling(H, V):
 
 def test_fastemit_and_clamp():
     check(1, 3, 9, 6, 640, 130, lam=0.01, clamp=0.05)
+
+
+@pytest.mark.parametrize("activation", ["tanh", "sigmoid"])
+@pytest.mark.parametrize("H,V", [(256, 37), (640, 129), (320, 1025)])
+def test_tanh_and_sigmoid_joints(activation, H, V):
+    """The other two activations the reference's joint accepts (modules/rnnt.py:1762-1770).  The kernel's float
+    tanh / exp and the oracle's float64 ones round to different bf16 neighbours for a few hidden units in a
+    hundred thousand; at these sizes that moves a cost by well under the 1e-5 bar."""
+    check(V + H + len(activation), 3, 8, 5, H, V, lam=0.01, activation=activation)
+    f, g, W, bias, labels, al, ll = make_case(1, 1, 2, 2, H, V)
+    lab, ald, lld = dev_ints(labels, al, ll)
+    with pytest.raises(ValueError, match="Unsupported activation"):  # the reference's message, modules/rnnt.py:1763
+        joint_rnnt_loss(f.to(DEV), g.to(DEV), W.to(DEV), bias.to(DEV), lab, ald, lld, V - 1, activation="gelu")
 
 
 def test_full_lengths_no_bias_bf16_weights():

@@ -31,18 +31,19 @@ def dev_ints(*arrays):
     return [torch.tensor(np.asarray(a), dtype=torch.int64, device=DEV) for a in arrays]
 
 
-def check(seed, B, T, U, H, V, big_blanks, sigma=0.05, lam=0.0, clamp=0.0, blank=None):
+def check(seed, B, T, U, H, V, big_blanks, sigma=0.05, lam=0.0, clamp=0.0, blank=None, activation="relu"):
     NB = len(big_blanks)
     blank = V - 1 if blank is None else blank
     f, g, W, bias, labels, al, ll = make_case(seed, B, T, U, H, V, NB)
     labels = np.minimum(labels, max(blank - NB - 1, 0))
     gc = (np.random.RandomState(seed + 1000).rand(B) + 0.5).astype(np.float32)
     ref = oracle.joint_rnnt_loss(f.float().numpy(), g.float().numpy(), W.numpy(), bias.numpy(), labels, al, ll, blank,
-                                 lam, clamp, gc, big_blank_durations=big_blanks, sigma=sigma)  # fmt: skip
+                                 lam, clamp, gc, big_blank_durations=big_blanks, sigma=sigma, activation=activation)  # fmt: skip
     fd, gd = f.to(DEV).requires_grad_(True), g.to(DEV).requires_grad_(True)
     Wd, bd = W.to(DEV).requires_grad_(True), bias.to(DEV).requires_grad_(True)
     lab, ald, lld = dev_ints(labels, al, ll)
-    costs = joint_multiblank_loss(fd, gd, Wd, bd, lab, ald, lld, blank, big_blanks, sigma, lam, clamp)
+    costs = joint_multiblank_loss(fd, gd, Wd, bd, lab, ald, lld, blank, big_blanks, sigma, lam, clamp,
+                                  activation=activation)
     (costs * torch.tensor(gc, device=DEV)).sum().backward()
     torch.cuda.synchronize()
     np.testing.assert_allclose(costs.detach().cpu().numpy(), ref[0], rtol=1e-5)
@@ -95,3 +96,7 @@ def test_rejects_bad_arguments():
         joint_multiblank_forward(*args, 1, [2, 4])  # no room for two big blanks below blank = 1
     with pytest.raises(RuntimeError):
         joint_multiblank_forward(*args, 11, list(range(2, 11)))  # nine big blanks
+
+
+def test_sigmoid_joint():
+    check(5, 3, 8, 5, 384, 131, [2, 3], lam=0.01, activation="sigmoid")

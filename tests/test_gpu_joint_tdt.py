@@ -40,7 +40,7 @@ def dev_ints(*arrays):
 
 
 def check(seed, B, T, U, H, V, durations, sigma=0.05, lam=0.0, clamp=0.0, ragged=True, bias_on=True,
-          weight_dtype=torch.float32, dropout=0.0):  # fmt: skip
+          weight_dtype=torch.float32, dropout=0.0, activation="relu"):  # fmt: skip
     D = len(durations)
     f, g, W, bias, labels, al, ll = make_case(seed, B, T, U, H, V, D, ragged)
     gc = (np.random.RandomState(seed + 1000).rand(B) + 0.5).astype(np.float32)
@@ -50,13 +50,14 @@ def check(seed, B, T, U, H, V, durations, sigma=0.05, lam=0.0, clamp=0.0, ragged
     keep = joint_dropout_mask(B, T, U, H, dropout, rng_seed, DEV).cpu().numpy() if dropout else None
     ref = oracle.joint_rnnt_loss(f.float().numpy(), g.float().numpy(), Wq.float().numpy(),
                                  None if bq is None else bq.float().numpy(), labels, al, ll, V - 1, lam, clamp, gc,
-                                 keep_mask=keep, dropout_p=dropout, durations=durations, sigma=sigma)  # fmt: skip
+                                 keep_mask=keep, dropout_p=dropout, durations=durations, sigma=sigma,
+                                 activation=activation)  # fmt: skip
     fd, gd = f.to(DEV).requires_grad_(True), g.to(DEV).requires_grad_(True)
     Wd = Wq.to(DEV).requires_grad_(True)
     bd = None if bq is None else bq.to(DEV).requires_grad_(True)
     lab, ald, lld = dev_ints(labels, al, ll)
     costs = joint_tdt_loss(fd, gd, Wd, bd, lab, ald, lld, V - 1, durations, sigma, lam, clamp, dropout=dropout,
-                           seed=rng_seed)  # fmt: skip
+                           seed=rng_seed, activation=activation)  # fmt: skip
     (costs * torch.tensor(gc, device=DEV)).sum().backward()
     torch.cuda.synchronize()
     assert costs.dtype == torch.float32 and costs.shape == (B,)
@@ -210,3 +211,9 @@ def test_fused_sub_batches_give_the_same_costs_and_gradients(tdt):
         assert (x - y).abs().max().item() <= 2.0**-7 * x.abs().max().item()
     with pytest.raises(ValueError):
         run(-1)
+
+
+@pytest.mark.parametrize("activation", ["tanh", "sigmoid"])
+def test_tanh_and_sigmoid_joints_with_dropout(activation):
+    """modules/rnnt.py:1762-1776: activation, then Dropout, then the Linear layer."""
+    check(77, 3, 9, 5, 640, 130, [0, 1, 2], lam=0.01, dropout=0.2, activation=activation)

@@ -41,6 +41,30 @@ def test_against_torch_autograd(shape):
         np.testing.assert_allclose(got, want, rtol=1e-9, atol=1e-11)
 
 
+@pytest.mark.parametrize("activation", ["tanh", "sigmoid"])
+def test_tanh_and_sigmoid_joints_against_torch_autograd(activation):
+    """The reference's joint may use tanh or sigmoid (modules/rnnt.py:1762-1770).  Exactly: torch's own activation with
+    its output rounded to bf16 and the slope taken at the rounded output.  Loosely (1 %, the size of a bf16 rounding
+    step on every slope): plain float64 autograd that knows nothing of that convention -- a wrong derivative or a
+    slope taken at the wrong place would be off by tens of percent."""
+    B, T, U, H, V = 2, 3, 4, 16, 7
+    rng = np.random.RandomState(31)
+    f, g = bf16_round(rng.randn(B, T, H)), bf16_round(rng.randn(B, U, H))
+    w, bias = bf16_round(rng.randn(V, H) / np.sqrt(H)), bf16_round(rng.randn(V))
+    labels = rng.randint(0, V - 1, size=(B, U - 1))
+    gc = rng.rand(B) + 0.5
+    got = oracle.joint_rnnt_loss(f, g, w, bias, labels, [T] * B, [U - 1] * B, V - 1, grad_costs=gc, activation=activation)
+    ref = joint_autograd(f, g, w, bias, labels, V - 1, gc, activation=activation)
+    for a, b in zip(got, ref):
+        np.testing.assert_allclose(a, b, rtol=1e-9, atol=1e-11)
+    loose = joint_autograd(f, g, w, bias, labels, V - 1, gc, activation=activation, rounded_activation=False)
+    np.testing.assert_allclose(got[0], loose[0], rtol=2e-3)
+    for a, b in zip(got[1:], loose[1:]):
+        assert np.abs(a - b).max() <= 2e-2 * np.abs(b).max()
+    with pytest.raises(ValueError):
+        oracle.joint_rnnt_loss(f, g, w, bias, labels, [T] * B, [U - 1] * B, V - 1, activation="gelu")
+
+
 def test_ragged_lengths_are_the_trimmed_problems():
     B, T, U, H, V = 3, 5, 4, 16, 9
     rng = np.random.RandomState(7)
