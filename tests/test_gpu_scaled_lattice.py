@@ -137,3 +137,29 @@ def test_minus_infinity_logits_take_the_log_route():
     logd = run(x, labels, al, ll, V - 1)
     assert np.array_equal(got["costs"], logd["costs"], equal_nan=True)
     assert np.array_equal(got["grads"][0], logd["grads"][0], equal_nan=True)
+
+
+def test_north_star_shape_scaled_against_log_domain():
+    """The benchmark configuration at full size (B=16, T=375, U=121, V=1025, ragged lengths): every utterance stays in
+    the scaled format and costs / gradients agree with the log-domain kernel far inside the bar of the task."""
+    from speech_amd import RNNTLossNumba, synthetic
+
+    cfg, acts, labels, act_lens, label_lens = synthetic.make_inputs(1, device=torch.device(DEV), generate_on_device=True)
+    B, T, U, V = acts.shape
+    loss = RNNTLossNumba(blank=cfg.blank, reduction="none", fastemit_lambda=0.001, clamp=0.0)
+    out = {}
+    for mode in (2, 1):
+        rnnt.set_lattice_mode(mode)
+        x = acts.detach().clone().requires_grad_(True)
+        costs = loss(x, labels, act_lens, label_lens)
+        costs.sum().backward()
+        out[mode] = (costs.detach().double().cpu().numpy(), x.grad)
+    # the formats the scaled run ended in, read from a workspace of its own
+    rnnt.set_lattice_mode(2)
+    ws = rnnt.new_workspace(acts)
+    c = torch.empty(B, dtype=torch.float32, device=acts.device)
+    rnnt.rnnt_forward(acts.detach(), labels, act_lens, label_lens, c, cfg.blank, 0.001, True, ws)
+    assert (rnnt.lattice_formats(ws, B, T, U).cpu().numpy() == 1).all()
+    np.testing.assert_allclose(out[2][0], out[1][0], rtol=1e-6)
+    np.testing.assert_allclose(c.double().cpu().numpy(), out[1][0], rtol=1e-6)
+    assert float((out[2][1] - out[1][1]).abs().max()) < 2e-6
