@@ -42,7 +42,7 @@ HBM_PEAK_GBPS = 8000.0  # MI355X HBM3E, published peak
 # (summaries under profiles/).  None = not measured for that workload.
 MEASURED_TRAFFIC_BYTES = {
     # profiles/transducer_kernels_cfg2_hbm_traffic.md: fetch 1.6477 GB + write 2.9802 GB
-    ("cfg2_rnnt_B16_T375_U121_V1025_f32", False): int((804542 * 2.0 + 2910372) * 1024),
+    ("cfg2_rnnt_B16_T375_U121_V1025_f32", False): int((804539 * 2.0 + 2910378) * 1024),
 }
 
 
