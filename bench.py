@@ -217,7 +217,7 @@ def graph_replay(torch, cfg, acts, labels, act_lens, label_lens, steps):
 def other_workloads(torch, dev, indices, steps=8, warmup=3):
     """The remaining benchmark configurations, a few steps each, outside the headline's timed region: median step
     time by stream events, algorithmic bytes and the fraction of the HBM peak of the whole fwd+bwd step."""
-    from speech_amd import MultiblankRNNTLossNumba, RNNTLossNumba, TDTLossNumba, synthetic
+    from speech_amd import MultiblankRNNTLossNumba, RNNTLossNumba, TDTLossNumba, _native, synthetic
 
     out = []
     for index in indices:
@@ -253,11 +253,22 @@ def other_workloads(torch, dev, indices, steps=8, warmup=3):
         assert bool(torch.isfinite(costs.float()).all()), "non-finite costs"
         per_step = sorted(marks[i].elapsed_time(marks[i + 1]) for i in range(steps))
         ms = 0.5 * (per_step[(steps - 1) // 2] + per_step[steps // 2])
+        # a second pass with every pipeline kernel bracketed by events (not part of ms_per_step: the brackets cost
+        # queue time): where the step goes, and how close the dominant kernel, the gradient pass, is to the HBM peak
+        _native.profile_enable(steps)
+        for _ in range(steps):
+            step()
+        torch.cuda.synchronize()
+        kernels = {k: v[0] / max(v[1], 1) for k, v in _native.profile_read().items()}
+        _native.profile_disable()
+        grad_ms = kernels.get("gradient_pass", 0.0)
         out.append({
             "workload": cfg.name, "steps": steps, "ms_per_step": ms, "logit_elems_per_s": cfg.elems / (ms * 1e-3),
             "algorithmic_bytes": nbytes["total"], "achieved_GBps": nbytes["total"] / (ms * 1e-3) / 1e9,
             "frac_of_peak": nbytes["total"] / (ms * 1e-3) / 1e9 / HBM_PEAK_GBPS,
             "dtype": {torch.float32: "f32", torch.bfloat16: "bf16", torch.float16: "f16"}[cfg.dtype],
+            "kernel_ms": kernels,
+            "gradient_pass_frac_of_peak": (nbytes["grad_stream"] / (grad_ms * 1e-3) / 1e9 / HBM_PEAK_GBPS) if grad_ms else None,
         })  # fmt: skip
         del acts, costs, loss
         torch.cuda.empty_cache()
