@@ -64,10 +64,17 @@ int mi_transducer_workspace_bytes(int B, int T, int U, int D, size_t* out_bytes)
  * utils/cuda_utils/gpu_rnnt_kernel.py:73-172; compute_costs_data,
  * utils/rnnt_helper.py:106-116).  with_betas != 0 also runs the backward variables
  * (compute_betas_kernel, gpu_rnnt_kernel.py:175-269), which mi_rnnt_backward needs;
- * with_betas == 0 is the reference's score_forward (gpu_rnnt.py:250-265). */
+ * with_betas == 0 is the reference's score_forward (gpu_rnnt.py:250-265).
+ * prefill_grads (nullable; the forward calls of all three losses take it): the buffer, of the shape and dtype of
+ * acts, that this call's backward call will write the gradient into.  The lattice recursion keeps a few dozen
+ * compute units busy and leaves HBM idle; given the buffer, the lattice launch carries extra workgroups that
+ * zero-fill the gradient of padded cells meanwhile (part of what zeros_like + `grads *= 0` do up front in the
+ * reference, rnnt_pytorch.py:58, gpu_rnnt.py:156), stop when the lattice ends, and record in the workspace how far
+ * they got.  The backward call is then given padding_zeroed = 2.  Ignored when with_betas == 0. */
 int mi_rnnt_forward(const void* acts, int act_dtype, const int64_t* labels, const int64_t* act_lens,
                     const int64_t* label_lens, float* costs, int B, int T, int U, int V, int blank,
-                    float fastemit_lambda, int with_betas, void* workspace, size_t workspace_bytes, void* stream);
+                    float fastemit_lambda, int with_betas, void* prefill_grads, void* workspace,
+                    size_t workspace_bytes, void* stream);
 
 /* RNNT backward: writes every element of grads[B,T,U,V] (same dtype as acts): the
  * gradient of costs[b] w.r.t. the logits for valid cells, FastEmit and clamp folded
@@ -79,8 +86,10 @@ int mi_rnnt_forward(const void* acts, int act_dtype, const int64_t* labels, cons
  * broadcast grad_output is stride 0) and the 'mean' reduction's 1/B (rnnt_pytorch.py:77-81)
  * into the same pass.  grad_scale: device float32, nullable; grad_scale_stride >= 0 in elements.
  * Must follow mi_rnnt_forward(with_betas != 0) on the same workspace and inputs.
- * padding_zeroed != 0: the padded cells of grads were already zero-filled by
- * mi_transducer_zero_padding (the caller made this call wait for it); they are then skipped. */
+ * padding_zeroed (the backward calls of all three losses take it): 0 = this call writes every padded cell;
+ * 1 = the padded cells of grads were already zero-filled by mi_transducer_zero_padding (the caller made this
+ * call wait for it) and are skipped; 2 = the forward call on this workspace was given these grads as
+ * prefill_grads, and the padded cells it reports as zero-filled are skipped.  Any other value is invalid. */
 int mi_rnnt_backward(const void* acts, int act_dtype, const int64_t* labels, const int64_t* act_lens,
                      const int64_t* label_lens, void* grads, const float* grad_scale, int grad_scale_stride,
                      float grad_mul, int padding_zeroed, int B, int T, int U, int V, int blank,
@@ -125,7 +134,7 @@ int mi_rnnt_loss_static(const void* acts, int act_dtype, const int64_t* labels, 
 int mi_tdt_forward(const void* acts, int act_dtype, const int64_t* labels, const int64_t* act_lens,
                    const int64_t* label_lens, float* costs, int B, int T, int U, int V, int D,
                    const int32_t* durations_host, int blank, float fastemit_lambda, float sigma, int use_plain_rnnt,
-                   int with_betas, void* workspace, size_t workspace_bytes, void* stream);
+                   int with_betas, void* prefill_grads, void* workspace, size_t workspace_bytes, void* stream);
 
 int mi_tdt_backward(const void* acts, int act_dtype, const int64_t* labels, const int64_t* act_lens,
                     const int64_t* label_lens, void* grads, const float* grad_scale, int grad_scale_stride,
@@ -147,16 +156,19 @@ int mi_tdt_loss(const void* acts, int act_dtype, const int64_t* labels, const in
  * arcs of each duration (gpu_rnnt_kernel.py:1328-1341; no clamp, no FastEmit on these); padded cells get zeros in
  * both.  use_plain_rnnt != 0 (the omega branch): plain RNNT on the token logits, duration_grads all zero.
  * The workspace is mi_transducer_workspace_bytes(B, T, U, D).  In mi_tdt_split_loss both gradient pointers are
- * given or both are NULL (forward only). */
+ * given or both are NULL (forward only).  prefill_label_grads / padding_zeroed: as for RNNT, on label_grads (the
+ * duration gradient is written by a kernel of its own, padded cells included). */
 int mi_tdt_split_forward(const void* label_acts, const void* duration_acts, int act_dtype, const int64_t* labels,
                          const int64_t* act_lens, const int64_t* label_lens, float* costs, int B, int T, int U, int V,
                          int D, const int32_t* durations_host, int blank, float fastemit_lambda, float sigma,
-                         int use_plain_rnnt, int with_betas, void* workspace, size_t workspace_bytes, void* stream);
+                         int use_plain_rnnt, int with_betas, void* prefill_label_grads, void* workspace,
+                         size_t workspace_bytes, void* stream);
 int mi_tdt_split_backward(const void* label_acts, int act_dtype, const int64_t* labels, const int64_t* act_lens,
                           const int64_t* label_lens, void* label_grads, void* duration_grads,
-                          const float* grad_scale, int grad_scale_stride, float grad_mul, int B, int T, int U, int V,
-                          int D, const int32_t* durations_host, int blank, float fastemit_lambda, float clamp,
-                          float sigma, int use_plain_rnnt, void* workspace, size_t workspace_bytes, void* stream);
+                          const float* grad_scale, int grad_scale_stride, float grad_mul, int padding_zeroed, int B,
+                          int T, int U, int V, int D, const int32_t* durations_host, int blank, float fastemit_lambda,
+                          float clamp, float sigma, int use_plain_rnnt, void* workspace, size_t workspace_bytes,
+                          void* stream);
 int mi_tdt_split_loss(const void* label_acts, const void* duration_acts, int act_dtype, const int64_t* labels,
                       const int64_t* act_lens, const int64_t* label_lens, float* costs, void* label_grads,
                       void* duration_grads, const float* grad_scale, int grad_scale_stride, float grad_mul, int B,
@@ -177,11 +189,11 @@ int mi_tdt_split_loss(const void* label_acts, const void* duration_acts, int act
 int mi_multiblank_forward(const void* acts, int act_dtype, const int64_t* labels, const int64_t* act_lens,
                           const int64_t* label_lens, float* costs, int B, int T, int U, int V, int num_big_blanks,
                           const int32_t* big_blank_durations_host, int blank, float fastemit_lambda, float sigma,
-                          int with_betas, void* workspace, size_t workspace_bytes, void* stream);
+                          int with_betas, void* prefill_grads, void* workspace, size_t workspace_bytes, void* stream);
 
 int mi_multiblank_backward(const void* acts, int act_dtype, const int64_t* labels, const int64_t* act_lens,
                            const int64_t* label_lens, void* grads, const float* grad_scale, int grad_scale_stride,
-                           float grad_mul, int B, int T, int U, int V, int num_big_blanks,
+                           float grad_mul, int padding_zeroed, int B, int T, int U, int V, int num_big_blanks,
                            const int32_t* big_blank_durations_host, int blank, float fastemit_lambda, float clamp,
                            float sigma, void* workspace, size_t workspace_bytes, void* stream);
 

@@ -21,7 +21,7 @@ CPU_SOURCES = [os.path.join(CSRC_DIR, "mi_cpu.cpp")]
 CPU_ABI_VERSION = 1
 CXX_FLAGS = ["-O3", "-std=c++17", "-fPIC", "-shared", "-fopenmp", "-Wall", "-Wextra"]
 
-ABI_VERSION = 16
+ABI_VERSION = 17
 SUCCESS, INVALID_VALUE, LAUNCH_FAILURE, TOO_LARGE = 0, 1, 2, 3
 STATIC_WORKSPACE_BYTES = 64 << 20
 DTYPE_F32, DTYPE_BF16, DTYPE_F16 = 0, 1, 2
@@ -75,7 +75,7 @@ _SIGNATURES = {
     "mi_transducer_abi_version": [],
     "mi_transducer_workspace_bytes": [_c_int, _c_int, _c_int, _c_int, ctypes.POINTER(_c_size_t)],
     "mi_rnnt_forward": [_vp, _c_int, _vp, _vp, _vp, _vp, _c_int, _c_int, _c_int, _c_int, _c_int, _c_float, _c_int,
-                        _vp, _c_size_t, _vp],
+                        _vp, _vp, _c_size_t, _vp],
     "mi_rnnt_backward": [_vp, _c_int, _vp, _vp, _vp, _vp, _vp, _c_int, _c_float, _c_int, _c_int, _c_int, _c_int,
                          _c_int, _c_int, _c_float, _c_float, _vp, _c_size_t, _vp],
     "mi_rnnt_loss": [_vp, _c_int, _vp, _vp, _vp, _vp, _vp, _vp, _c_int, _c_float, _c_int, _c_int, _c_int, _c_int,
@@ -84,21 +84,22 @@ _SIGNATURES = {
     "mi_rnnt_loss_static": [_vp, _c_int, _vp, _vp, _vp, _vp, _vp, _vp, _c_int, _c_float, _c_int, _c_int, _c_int, _c_int,
                             _c_int, _c_float, _c_float, _vp],
     "mi_tdt_forward": [_vp, _c_int, _vp, _vp, _vp, _vp, _c_int, _c_int, _c_int, _c_int, _c_int, _vp, _c_int, _c_float,
-                       _c_float, _c_int, _c_int, _vp, _c_size_t, _vp],
+                       _c_float, _c_int, _c_int, _vp, _vp, _c_size_t, _vp],
     "mi_tdt_backward": [_vp, _c_int, _vp, _vp, _vp, _vp, _vp, _c_int, _c_float, _c_int, _c_int, _c_int, _c_int,
                         _c_int, _c_int, _vp, _c_int, _c_float, _c_float, _c_float, _c_int, _vp, _c_size_t, _vp],
     "mi_tdt_loss": [_vp, _c_int, _vp, _vp, _vp, _vp, _vp, _vp, _c_int, _c_float, _c_int, _c_int, _c_int, _c_int,
                     _c_int, _vp, _c_int, _c_float, _c_float, _c_float, _c_int, _vp, _c_size_t, _vp],
     "mi_tdt_split_forward": [_vp, _vp, _c_int, _vp, _vp, _vp, _vp, _c_int, _c_int, _c_int, _c_int, _c_int, _vp, _c_int,
-                             _c_float, _c_float, _c_int, _c_int, _vp, _c_size_t, _vp],
+                             _c_float, _c_float, _c_int, _c_int, _vp, _vp, _c_size_t, _vp],
     "mi_tdt_split_backward": [_vp, _c_int, _vp, _vp, _vp, _vp, _vp, _vp, _c_int, _c_float, _c_int, _c_int, _c_int,
-                              _c_int, _c_int, _vp, _c_int, _c_float, _c_float, _c_float, _c_int, _vp, _c_size_t, _vp],
+                              _c_int, _c_int, _c_int, _vp, _c_int, _c_float, _c_float, _c_float, _c_int, _vp,
+                              _c_size_t, _vp],
     "mi_tdt_split_loss": [_vp, _vp, _c_int, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _c_int, _c_float, _c_int, _c_int, _c_int,
                           _c_int, _c_int, _vp, _c_int, _c_float, _c_float, _c_float, _c_int, _vp, _c_size_t, _vp],
     "mi_multiblank_forward": [_vp, _c_int, _vp, _vp, _vp, _vp, _c_int, _c_int, _c_int, _c_int, _c_int, _vp, _c_int,
-                              _c_float, _c_float, _c_int, _vp, _c_size_t, _vp],
+                              _c_float, _c_float, _c_int, _vp, _vp, _c_size_t, _vp],
     "mi_multiblank_backward": [_vp, _c_int, _vp, _vp, _vp, _vp, _vp, _c_int, _c_float, _c_int, _c_int, _c_int, _c_int,
-                               _c_int, _vp, _c_int, _c_float, _c_float, _c_float, _vp, _c_size_t, _vp],
+                               _c_int, _c_int, _vp, _c_int, _c_float, _c_float, _c_float, _vp, _c_size_t, _vp],
     "mi_multiblank_loss": [_vp, _c_int, _vp, _vp, _vp, _vp, _vp, _vp, _c_int, _c_float, _c_int, _c_int, _c_int, _c_int,
                            _c_int, _vp, _c_int, _c_float, _c_float, _c_float, _vp, _c_size_t, _vp],
     "mi_rnnt_logprobs_forward": [_vp, _c_int, _vp, _vp, _vp, _vp, _vp, _c_int, _c_int, _c_int, _c_int, _c_int, _vp,

@@ -25,6 +25,29 @@ constexpr int kScaleFormat = 4;  // index of the format word in the header
 constexpr int kScaleBlock = 8;
 constexpr int kScaleMaxBlocks = 2048;  // exponent tracks the scaled lattice kernel can hold in LDS
 
+// The prefill segment of the workspace, in ints.  While a lattice kernel runs, HBM idles; "riders" (extra workgroups
+// of the same launch) zero-fill the padded cells of the gradient meanwhile, as far as they get.
+//   [0, kFillMaxLattice)                  per lattice workgroup: (epoch << 13) | (id of the compute unit it runs on + 1)
+//   [kFillMaxLattice, 2*kFillMaxLattice)  per lattice workgroup: the epoch, once it has finished
+//   [2*kFillMaxLattice, + kFillMaxRiders) per virtual rider: how many of its items have been filled
+// An item is 2^prefill_log_rows rows of one frame (b, t), items are numbered in memory order, and item i is the
+// (i / kFillMaxRiders)-th item of virtual rider i % kFillMaxRiders: it is done iff  i / kFillMaxRiders <
+// progress[i % kFillMaxRiders].  A launch has a power of two of real riders, each standing for the virtual riders
+// congruent to it.  The epoch changes with every launch: what an earlier call left in the first two blocks is not
+// mistaken for this call's.
+constexpr int kFillMaxLattice = 256;
+constexpr int kFillMaxRiders = 4096;
+constexpr int kFillProgress = 2 * kFillMaxLattice;
+constexpr int kFillInts = kFillProgress + kFillMaxRiders;
+constexpr int kFillLogRowsShift = 8;  // the gradient kernels find log2(rows per item) in these bits of `flags`
+// Rows per item: eight (no workgroup of the gradient pass spans more rows, and none straddles a multiple of eight),
+// fewer for long rows, so that a rider looks at the lattice's state every 64 KB or so
+inline int prefill_log_rows(size_t row_bytes) {
+  int log_rows = 3;
+  while (log_rows > 0 && (row_bytes << log_rows) > 64 * 1024) --log_rows;
+  return log_rows;
+}
+
 // ----------------------------------------------------------------------------------------
 // Workspace layout
 // ----------------------------------------------------------------------------------------
@@ -35,7 +58,7 @@ struct Layout {
   int A;    // arc planes per diagonal row: blank, label, D duration log-probs
   int CS;   // floats per cell in the coefficient buffer
   int SG;   // ints per utterance in the scale segment: kScaleHeader, then {alpha, beta} exponent per 8 diagonals
-  size_t off_denom, off_arcs, off_alphas, off_betas, off_ll, off_coef, off_scale, total;
+  size_t off_denom, off_arcs, off_alphas, off_betas, off_ll, off_coef, off_scale, off_fill, total;
   size_t off_arcp, total_scaled;  // total_scaled = total + the arc-probability segment of the scaled RNNT lattice
 };
 
@@ -63,6 +86,7 @@ inline bool make_layout(int B, int T, int U, int D, Layout* L) {
   // of the alpha and beta values of every block of kScaleBlock anti-diagonals of a scaled lattice
   L->SG = kScaleHeader + 2 * ((L->ND / kScaleBlock + 3) & ~1);
   L->off_scale = off;  off = align256(off + (size_t)B * L->SG * sizeof(int));
+  L->off_fill = off;   off = align256(off + (size_t)kFillInts * sizeof(int));
   L->total = off;
   // the scaled (probability-domain) RNNT lattice also wants the blank / label arc PROBABILITIES as doubles, skewed
   // like `arcs`: a segment behind everything else that only a caller who asked for that lattice has to bring

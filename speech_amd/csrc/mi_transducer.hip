@@ -48,6 +48,7 @@ namespace {
 
 #include "mi_plan.h"
 #include "mi_device.inc"
+#include "mi_prefill.inc"
 #include "mi_lattice.inc"
 #include "mi_logprobs.inc"
 #include "mi_multiblank.inc"
@@ -64,7 +65,7 @@ namespace {
 // ----------------------------------------------------------------------------------------
 extern "C" {
 
-int mi_transducer_abi_version(void) { return 16; }
+int mi_transducer_abi_version(void) { return 17; }
 
 int mi_transducer_workspace_bytes(int B, int T, int U, int D, size_t* out_bytes) {
   Layout L;
@@ -76,7 +77,8 @@ int mi_transducer_workspace_bytes(int B, int T, int U, int D, size_t* out_bytes)
 
 int mi_rnnt_forward(const void* acts, int act_dtype, const int64_t* labels, const int64_t* act_lens,
                     const int64_t* label_lens, float* costs, int B, int T, int U, int V, int blank,
-                    float fastemit_lambda, int with_betas, void* workspace, size_t workspace_bytes, void* stream) {
+                    float fastemit_lambda, int with_betas, void* prefill_grads, void* workspace,
+                    size_t workspace_bytes, void* stream) {
   Common c;
   if (!costs) return MI_TRANSDUCER_INVALID_VALUE;
   int st = check_common(acts, act_dtype, labels, act_lens, label_lens, B, T, U, V, 0, blank, workspace,
@@ -84,7 +86,7 @@ int mi_rnnt_forward(const void* acts, int act_dtype, const int64_t* labels, cons
   if (st) return st;
   const unsigned long long mark = scaled_lattice_mark(c, with_betas);
   if ((st = run_denom(c, mark))) return st;
-  return run_rnnt_lattice(c, costs, fastemit_lambda, with_betas, mark);
+  return run_rnnt_lattice(c, costs, fastemit_lambda, with_betas, mark, with_betas ? prefill_grads : nullptr);
 }
 
 int mi_rnnt_backward(const void* acts, int act_dtype, const int64_t* labels, const int64_t* act_lens,
@@ -92,25 +94,27 @@ int mi_rnnt_backward(const void* acts, int act_dtype, const int64_t* labels, con
                      float grad_mul, int padding_zeroed, int B, int T, int U, int V, int blank,
                      float fastemit_lambda, float clamp, void* workspace, size_t workspace_bytes, void* stream) {
   Common c;
-  if (!grads || clamp < 0.f || grad_scale_stride < 0) return MI_TRANSDUCER_INVALID_VALUE;
+  if (!grads || clamp < 0.f || grad_scale_stride < 0 || padding_zeroed < 0 || padding_zeroed > 2)
+    return MI_TRANSDUCER_INVALID_VALUE;
   int st = check_common(acts, act_dtype, labels, act_lens, label_lens, B, T, U, V, 0, blank, workspace,
                         workspace_bytes, stream, &c);
   if (st) return st;
   const ScaleArg sc = {grad_scale, grad_scale_stride, grad_mul};
   const bool fused = rnnt_rows_fused(c, grads);
   if (!fused && (st = run_rnnt_cells(c, sc, fastemit_lambda, clamp))) return st;
-  return run_grad_stream(c, grads, padding_zeroed ? kFlagPaddingDone : 0, fused, sc, fastemit_lambda, clamp);
+  return run_grad_stream(c, grads, padding_flags(padding_zeroed), fused, sc, fastemit_lambda, clamp);
 }
 
 int mi_rnnt_loss(const void* acts, int act_dtype, const int64_t* labels, const int64_t* act_lens,
                  const int64_t* label_lens, float* costs, void* grads, const float* grad_scale,
                  int grad_scale_stride, float grad_mul, int B, int T, int U, int V, int blank, float fastemit_lambda,
                  float clamp, void* workspace, size_t workspace_bytes, void* stream) {
+  // (the lattice launch zero-fills padded cells of grads while it runs; the gradient pass skips those)
   int st = mi_rnnt_forward(acts, act_dtype, labels, act_lens, label_lens, costs, B, T, U, V, blank, fastemit_lambda,
-                           grads != nullptr, workspace, workspace_bytes, stream);
+                           grads != nullptr, grads, workspace, workspace_bytes, stream);
   if (st || !grads) return st;
   return mi_rnnt_backward(acts, act_dtype, labels, act_lens, label_lens, grads, grad_scale, grad_scale_stride,
-                          grad_mul, 0, B, T, U, V, blank, fastemit_lambda, clamp, workspace, workspace_bytes, stream);
+                          grad_mul, 2, B, T, U, V, blank, fastemit_lambda, clamp, workspace, workspace_bytes, stream);
 }
 
 // ----------------------------------------------------------------------------------------
@@ -167,10 +171,11 @@ int mi_rnnt_loss_static(const void* acts, int act_dtype, const int64_t* labels, 
 int mi_tdt_forward(const void* acts, int act_dtype, const int64_t* labels, const int64_t* act_lens,
                    const int64_t* label_lens, float* costs, int B, int T, int U, int V, int D,
                    const int32_t* durations_host, int blank, float fastemit_lambda, float sigma, int use_plain_rnnt,
-                   int with_betas, void* workspace, size_t workspace_bytes, void* stream) {
+                   int with_betas, void* prefill_grads, void* workspace, size_t workspace_bytes, void* stream) {
   Common c;
   TdtParams prm;
   if (!costs) return MI_TRANSDUCER_INVALID_VALUE;
+  if (!with_betas) prefill_grads = nullptr;
   int st = make_tdt_params(D, durations_host, sigma, &prm);
   if (st) return st;
   st = check_common(acts, act_dtype, labels, act_lens, label_lens, B, T, U, V, D, blank, workspace, workspace_bytes,
@@ -178,8 +183,8 @@ int mi_tdt_forward(const void* acts, int act_dtype, const int64_t* labels, const
   if (st) return st;
   if ((st = run_denom(c))) return st;
   // omega branch (gpu_rnnt.py:607-622): the plain RNNT recursion over the token logits
-  if (use_plain_rnnt) return run_rnnt_lattice(c, costs, fastemit_lambda, with_betas);
-  return run_tdt_lattice(c, costs, fastemit_lambda, with_betas, prm);
+  if (use_plain_rnnt) return run_rnnt_lattice(c, costs, fastemit_lambda, with_betas, 0, prefill_grads);
+  return run_tdt_lattice(c, costs, fastemit_lambda, with_betas, prm, prefill_grads);
 }
 
 int mi_tdt_backward(const void* acts, int act_dtype, const int64_t* labels, const int64_t* act_lens,
@@ -189,8 +194,9 @@ int mi_tdt_backward(const void* acts, int act_dtype, const int64_t* labels, cons
                     int use_plain_rnnt, void* workspace, size_t workspace_bytes, void* stream) {
   Common c;
   TdtParams prm;
-  if (!grads || clamp < 0.f || grad_scale_stride < 0) return MI_TRANSDUCER_INVALID_VALUE;
-  const int pad_flag = padding_zeroed ? kFlagPaddingDone : 0;
+  if (!grads || clamp < 0.f || grad_scale_stride < 0 || padding_zeroed < 0 || padding_zeroed > 2)
+    return MI_TRANSDUCER_INVALID_VALUE;
+  const int pad_flag = padding_flags(padding_zeroed);
   int st = make_tdt_params(D, durations_host, sigma, &prm);
   if (st) return st;
   st = check_common(acts, act_dtype, labels, act_lens, label_lens, B, T, U, V, D, blank, workspace, workspace_bytes,
@@ -211,40 +217,48 @@ int mi_tdt_loss(const void* acts, int act_dtype, const int64_t* labels, const in
                 float grad_mul, int B, int T, int U, int V, int D, const int32_t* durations_host, int blank,
                 float fastemit_lambda, float clamp, float sigma, int use_plain_rnnt, void* workspace,
                 size_t workspace_bytes, void* stream) {
+  void* prefill = grads;
   int st = mi_tdt_forward(acts, act_dtype, labels, act_lens, label_lens, costs, B, T, U, V, D, durations_host, blank,
-                          fastemit_lambda, sigma, use_plain_rnnt, grads != nullptr, workspace, workspace_bytes, stream);
+                          fastemit_lambda, sigma, use_plain_rnnt, grads != nullptr, prefill, workspace, workspace_bytes,
+                          stream);
   if (st || !grads) return st;
   return mi_tdt_backward(acts, act_dtype, labels, act_lens, label_lens, grads, grad_scale, grad_scale_stride, grad_mul,
-                         0, B, T, U, V, D, durations_host, blank, fastemit_lambda, clamp, sigma, use_plain_rnnt,
-                         workspace, workspace_bytes, stream);
+                         prefill ? 2 : 0, B, T, U, V, D, durations_host, blank, fastemit_lambda, clamp, sigma,
+                         use_plain_rnnt, workspace, workspace_bytes, stream);
 }
 
 int mi_tdt_split_forward(const void* label_acts, const void* duration_acts, int act_dtype, const int64_t* labels,
                          const int64_t* act_lens, const int64_t* label_lens, float* costs, int B, int T, int U, int V,
                          int D, const int32_t* durations_host, int blank, float fastemit_lambda, float sigma,
-                         int use_plain_rnnt, int with_betas, void* workspace, size_t workspace_bytes, void* stream) {
+                         int use_plain_rnnt, int with_betas, void* prefill_label_grads, void* workspace,
+                         size_t workspace_bytes, void* stream) {
   Common c;
   TdtParams prm;
   if (!costs || !duration_acts) return MI_TRANSDUCER_INVALID_VALUE;
+  if (!with_betas) prefill_label_grads = nullptr;
   int st = make_tdt_params(D, durations_host, sigma, &prm);
   if (st) return st;
   st = check_common(label_acts, act_dtype, labels, act_lens, label_lens, B, T, U, V, 0, blank, workspace,
                     workspace_bytes, stream, &c, 0, D);
   if (st) return st;
   if ((st = run_denom(c))) return st;
-  if (use_plain_rnnt) return run_rnnt_lattice(c, costs, fastemit_lambda, with_betas);
+  if (use_plain_rnnt) return run_rnnt_lattice(c, costs, fastemit_lambda, with_betas, 0, prefill_label_grads);
   if ((st = run_tdt_duration_planes(c, duration_acts, D))) return st;
-  return run_tdt_lattice(c, costs, fastemit_lambda, with_betas, prm);
+  return run_tdt_lattice(c, costs, fastemit_lambda, with_betas, prm, prefill_label_grads);
 }
 
 int mi_tdt_split_backward(const void* label_acts, int act_dtype, const int64_t* labels, const int64_t* act_lens,
                           const int64_t* label_lens, void* label_grads, void* duration_grads,
-                          const float* grad_scale, int grad_scale_stride, float grad_mul, int B, int T, int U, int V,
-                          int D, const int32_t* durations_host, int blank, float fastemit_lambda, float clamp,
-                          float sigma, int use_plain_rnnt, void* workspace, size_t workspace_bytes, void* stream) {
+                          const float* grad_scale, int grad_scale_stride, float grad_mul, int padding_zeroed, int B,
+                          int T, int U, int V, int D, const int32_t* durations_host, int blank, float fastemit_lambda,
+                          float clamp, float sigma, int use_plain_rnnt, void* workspace, size_t workspace_bytes,
+                          void* stream) {
   Common c;
   TdtParams prm;
-  if (!label_grads || !duration_grads || clamp < 0.f || grad_scale_stride < 0) return MI_TRANSDUCER_INVALID_VALUE;
+  if (!label_grads || !duration_grads || clamp < 0.f || grad_scale_stride < 0 || padding_zeroed < 0 ||
+      padding_zeroed > 2)
+    return MI_TRANSDUCER_INVALID_VALUE;
+  const int pad_flag = padding_flags(padding_zeroed);
   int st = make_tdt_params(D, durations_host, sigma, &prm);
   if (st) return st;
   st = check_common(label_acts, act_dtype, labels, act_lens, label_lens, B, T, U, V, 0, blank, workspace,
@@ -254,11 +268,11 @@ int mi_tdt_split_backward(const void* label_acts, int act_dtype, const int64_t* 
   if (use_plain_rnnt) {  // gpu_rnnt.py:646-682: token gradient from the RNNT kernel, duration gradient stays zero
     const bool fused = rnnt_rows_fused(c, label_grads);
     if (!fused && (st = run_rnnt_cells(c, sc, fastemit_lambda, clamp))) return st;
-    if ((st = run_grad_stream(c, label_grads, 0, fused, sc, fastemit_lambda, clamp))) return st;
+    if ((st = run_grad_stream(c, label_grads, pad_flag, fused, sc, fastemit_lambda, clamp))) return st;
     return run_tdt_duration_grads(c, duration_grads, D, 1);
   }
   if ((st = run_tdt_cells(c, sc, fastemit_lambda, clamp, prm, 1))) return st;
-  if ((st = run_grad_stream(c, label_grads, 0, false, sc, fastemit_lambda, clamp))) return st;
+  if ((st = run_grad_stream(c, label_grads, pad_flag, false, sc, fastemit_lambda, clamp))) return st;
   return run_tdt_duration_grads(c, duration_grads, D, 0);
 }
 
@@ -269,39 +283,42 @@ int mi_tdt_split_loss(const void* label_acts, const void* duration_acts, int act
                       float clamp, float sigma, int use_plain_rnnt, void* workspace, size_t workspace_bytes,
                       void* stream) {
   if ((label_grads == nullptr) != (duration_grads == nullptr)) return MI_TRANSDUCER_INVALID_VALUE;
+  void* prefill = label_grads;
   int st = mi_tdt_split_forward(label_acts, duration_acts, act_dtype, labels, act_lens, label_lens, costs, B, T, U, V, D,
                                 durations_host, blank, fastemit_lambda, sigma, use_plain_rnnt, label_grads != nullptr,
-                                workspace, workspace_bytes, stream);
+                                prefill, workspace, workspace_bytes, stream);
   if (st || !label_grads) return st;
   return mi_tdt_split_backward(label_acts, act_dtype, labels, act_lens, label_lens, label_grads, duration_grads,
-                               grad_scale, grad_scale_stride, grad_mul, B, T, U, V, D, durations_host, blank,
-                               fastemit_lambda, clamp, sigma, use_plain_rnnt, workspace, workspace_bytes, stream);
+                               grad_scale, grad_scale_stride, grad_mul, prefill ? 2 : 0, B, T, U, V, D, durations_host,
+                               blank, fastemit_lambda, clamp, sigma, use_plain_rnnt, workspace, workspace_bytes, stream);
 }
 
 int mi_multiblank_forward(const void* acts, int act_dtype, const int64_t* labels, const int64_t* act_lens,
                           const int64_t* label_lens, float* costs, int B, int T, int U, int V, int num_big_blanks,
                           const int32_t* big_blank_durations_host, int blank, float fastemit_lambda, float sigma,
-                          int with_betas, void* workspace, size_t workspace_bytes, void* stream) {
+                          int with_betas, void* prefill_grads, void* workspace, size_t workspace_bytes, void* stream) {
   Common c;
   MbParams prm;
   if (!costs) return MI_TRANSDUCER_INVALID_VALUE;
+  if (!with_betas) prefill_grads = nullptr;
   int st = make_mb_params(num_big_blanks, big_blank_durations_host, sigma, &prm);
   if (st) return st;
   st = check_common(acts, act_dtype, labels, act_lens, label_lens, B, T, U, V, 0, blank, workspace, workspace_bytes,
                     stream, &c, num_big_blanks);
   if (st) return st;
   if ((st = run_denom(c))) return st;
-  return run_multiblank_lattice(c, costs, fastemit_lambda, with_betas, prm);
+  return run_multiblank_lattice(c, costs, fastemit_lambda, with_betas, prm, prefill_grads);
 }
 
 int mi_multiblank_backward(const void* acts, int act_dtype, const int64_t* labels, const int64_t* act_lens,
                            const int64_t* label_lens, void* grads, const float* grad_scale, int grad_scale_stride,
-                           float grad_mul, int B, int T, int U, int V, int num_big_blanks,
+                           float grad_mul, int padding_zeroed, int B, int T, int U, int V, int num_big_blanks,
                            const int32_t* big_blank_durations_host, int blank, float fastemit_lambda, float clamp,
                            float sigma, void* workspace, size_t workspace_bytes, void* stream) {
   Common c;
   MbParams prm;
-  if (!grads || clamp < 0.f || grad_scale_stride < 0) return MI_TRANSDUCER_INVALID_VALUE;
+  if (!grads || clamp < 0.f || grad_scale_stride < 0 || padding_zeroed < 0 || padding_zeroed > 2)
+    return MI_TRANSDUCER_INVALID_VALUE;
   int st = make_mb_params(num_big_blanks, big_blank_durations_host, sigma, &prm);
   if (st) return st;
   st = check_common(acts, act_dtype, labels, act_lens, label_lens, B, T, U, V, 0, blank, workspace, workspace_bytes,
@@ -309,7 +326,7 @@ int mi_multiblank_backward(const void* acts, int act_dtype, const int64_t* label
   if (st) return st;
   const ScaleArg sc = {grad_scale, grad_scale_stride, grad_mul};
   if ((st = run_multiblank_cells(c, sc, fastemit_lambda, clamp, prm))) return st;
-  if ((st = run_grad_stream(c, grads, 0, false, sc, fastemit_lambda, clamp))) return st;
+  if ((st = run_grad_stream(c, grads, padding_flags(padding_zeroed), false, sc, fastemit_lambda, clamp))) return st;
   return run_multiblank_fixup(c, grads, prm);
 }
 
@@ -319,11 +336,11 @@ int mi_multiblank_loss(const void* acts, int act_dtype, const int64_t* labels, c
                        const int32_t* big_blank_durations_host, int blank, float fastemit_lambda, float clamp,
                        float sigma, void* workspace, size_t workspace_bytes, void* stream) {
   int st = mi_multiblank_forward(acts, act_dtype, labels, act_lens, label_lens, costs, B, T, U, V, num_big_blanks,
-                                 big_blank_durations_host, blank, fastemit_lambda, sigma, grads != nullptr, workspace,
-                                 workspace_bytes, stream);
+                                 big_blank_durations_host, blank, fastemit_lambda, sigma, grads != nullptr, grads,
+                                 workspace, workspace_bytes, stream);
   if (st || !grads) return st;
   return mi_multiblank_backward(acts, act_dtype, labels, act_lens, label_lens, grads, grad_scale, grad_scale_stride,
-                                grad_mul, B, T, U, V, num_big_blanks, big_blank_durations_host, blank, fastemit_lambda,
+                                grad_mul, 2, B, T, U, V, num_big_blanks, big_blank_durations_host, blank, fastemit_lambda,
                                 clamp, sigma, workspace, workspace_bytes, stream);
 }
 

@@ -63,6 +63,15 @@ def _durations_array(durations):
     return arr, ctypes.cast(arr, ctypes.c_void_p)
 
 
+def _check_prefill(acts, prefill_grads):
+    if prefill_grads is None:
+        return
+    if prefill_grads.shape != acts.shape or prefill_grads.dtype != acts.dtype or prefill_grads.device != acts.device:
+        raise ValueError("prefill_grads must have the shape, dtype and device of acts")
+    if not prefill_grads.is_contiguous():
+        raise ValueError("prefill_grads must be contiguous")
+
+
 def new_workspace(acts, num_durations=0):
     """Scratch for one call (replaces torch.zeros(get_workspace_size(...)), rnnt.py:182-189; not zero-filled)."""
     B, T, U = acts.shape[:3]
@@ -131,13 +140,18 @@ def tdt_lattice(act_lens, label_lens, costs, B, T, U, durations, fastemit_lambda
     _native.check_status(status, "Could not calculate forward scores")
 
 
-def rnnt_forward(acts, labels, act_lens, label_lens, costs, blank, fastemit_lambda, with_betas, workspace):
+def rnnt_forward(acts, labels, act_lens, label_lens, costs, blank, fastemit_lambda, with_betas, workspace,
+                 prefill_grads=None):
+    """prefill_grads: the buffer (shape and dtype of acts) that the backward call of this forward call will write the
+    gradient into, or None.  While the lattice recursion runs, extra workgroups of its launch zero-fill the padded
+    cells of that buffer as far as they get; rnnt_backward(..., padding_zeroed=2) then skips what they did."""
     _require_gpu(acts, "rnnt_forward")
     B, T, U, V = acts.shape
+    _check_prefill(acts, prefill_grads)
     with torch.cuda.device(acts.device):
         status = _native.lib().mi_rnnt_forward(
             _ptr(acts), _dtype_code(acts), _labels_ptr(labels), _ptr(act_lens), _ptr(label_lens), _ptr(costs),
-            B, T, U, V, int(blank), float(fastemit_lambda), int(bool(with_betas)),
+            B, T, U, V, int(blank), float(fastemit_lambda), int(bool(with_betas)), _ptr(prefill_grads),
             _ptr(workspace), workspace.numel(), _stream(acts.device),
         )  # fmt: skip
     _native.check_status(status, "Could not calculate forward scores")
@@ -149,13 +163,13 @@ def rnnt_backward(
 ):  # fmt: skip
     """grad_scale: device float32 tensor read as grad_scale[b * grad_scale_stride] (or None); every gradient is
     additionally multiplied by the host scalar grad_mul.  padding_zeroed: zero_padding() already ran on grads
-    and the current stream waits for it."""
+    and the current stream waits for it (1), or the forward call was given grads as prefill_grads (2)."""
     _require_gpu(acts, "rnnt_backward")
     B, T, U, V = acts.shape
     with torch.cuda.device(acts.device):
         status = _native.lib().mi_rnnt_backward(
             _ptr(acts), _dtype_code(acts), _labels_ptr(labels), _ptr(act_lens), _ptr(label_lens), _ptr(grads),
-            _ptr(grad_scale), int(grad_scale_stride), float(grad_mul), int(bool(padding_zeroed)), B, T, U, V, int(blank),
+            _ptr(grad_scale), int(grad_scale_stride), float(grad_mul), int(padding_zeroed), B, T, U, V, int(blank),
             float(fastemit_lambda), float(clamp), _ptr(workspace), workspace.numel(), _stream(acts.device),
         )  # fmt: skip
     _native.check_status(status, "Could not calculate gradients")
@@ -163,17 +177,19 @@ def rnnt_backward(
 
 def tdt_forward(
     acts, labels, act_lens, label_lens, costs, blank, durations, fastemit_lambda, sigma, use_plain_rnnt, with_betas,
-    workspace,
+    workspace, prefill_grads=None,
 ):  # fmt: skip
+    """prefill_grads: as for rnnt_forward."""
     _require_gpu(acts, "tdt_forward")
     B, T, U, VD = acts.shape
+    _check_prefill(acts, prefill_grads)
     D = len(durations)
     keep, dur_ptr = _durations_array(durations)
     with torch.cuda.device(acts.device):
         status = _native.lib().mi_tdt_forward(
             _ptr(acts), _dtype_code(acts), _labels_ptr(labels), _ptr(act_lens), _ptr(label_lens), _ptr(costs),
             B, T, U, VD - D, D, dur_ptr, int(blank), float(fastemit_lambda), float(sigma), int(bool(use_plain_rnnt)),
-            int(bool(with_betas)), _ptr(workspace), workspace.numel(), _stream(acts.device),
+            int(bool(with_betas)), _ptr(prefill_grads), _ptr(workspace), workspace.numel(), _stream(acts.device),
         )  # fmt: skip
     del keep
     _native.check_status(status, "Could not calculate forward scores")
@@ -190,7 +206,7 @@ def tdt_backward(
     with torch.cuda.device(acts.device):
         status = _native.lib().mi_tdt_backward(
             _ptr(acts), _dtype_code(acts), _labels_ptr(labels), _ptr(act_lens), _ptr(label_lens), _ptr(grads),
-            _ptr(grad_scale), int(grad_scale_stride), float(grad_mul), int(bool(padding_zeroed)), B, T, U, VD - D, D,
+            _ptr(grad_scale), int(grad_scale_stride), float(grad_mul), int(padding_zeroed), B, T, U, VD - D, D,
             dur_ptr, int(blank), float(fastemit_lambda), float(clamp), float(sigma), int(bool(use_plain_rnnt)),
             _ptr(workspace), workspace.numel(), _stream(acts.device),
         )  # fmt: skip
@@ -199,16 +215,19 @@ def tdt_backward(
 
 
 def multiblank_forward(
-    acts, labels, act_lens, label_lens, costs, blank, big_blank_durations, fastemit_lambda, sigma, with_betas, workspace
-):
+    acts, labels, act_lens, label_lens, costs, blank, big_blank_durations, fastemit_lambda, sigma, with_betas, workspace,
+    prefill_grads=None,
+):  # fmt: skip
+    """prefill_grads: as for rnnt_forward."""
     _require_gpu(acts, "multiblank_forward")
     B, T, U, V = acts.shape
+    _check_prefill(acts, prefill_grads)
     keep, dur_ptr = _durations_array(big_blank_durations)
     with torch.cuda.device(acts.device):
         status = _native.lib().mi_multiblank_forward(
             _ptr(acts), _dtype_code(acts), _labels_ptr(labels), _ptr(act_lens), _ptr(label_lens), _ptr(costs),
             B, T, U, V, len(big_blank_durations), dur_ptr, int(blank), float(fastemit_lambda), float(sigma),
-            int(bool(with_betas)), _ptr(workspace), workspace.numel(), _stream(acts.device),
+            int(bool(with_betas)), _ptr(prefill_grads), _ptr(workspace), workspace.numel(), _stream(acts.device),
         )  # fmt: skip
     del keep
     _native.check_status(status, "Could not calculate forward scores")
@@ -216,7 +235,7 @@ def multiblank_forward(
 
 def multiblank_backward(
     acts, labels, act_lens, label_lens, grads, grad_scale, blank, big_blank_durations, fastemit_lambda, clamp, sigma,
-    workspace, grad_scale_stride=1, grad_mul=1.0,
+    workspace, grad_scale_stride=1, grad_mul=1.0, padding_zeroed=0,
 ):  # fmt: skip
     _require_gpu(acts, "multiblank_backward")
     B, T, U, V = acts.shape
@@ -224,7 +243,8 @@ def multiblank_backward(
     with torch.cuda.device(acts.device):
         status = _native.lib().mi_multiblank_backward(
             _ptr(acts), _dtype_code(acts), _labels_ptr(labels), _ptr(act_lens), _ptr(label_lens), _ptr(grads),
-            _ptr(grad_scale), int(grad_scale_stride), float(grad_mul), B, T, U, V, len(big_blank_durations), dur_ptr,
+            _ptr(grad_scale), int(grad_scale_stride), float(grad_mul), int(padding_zeroed), B, T, U, V,
+            len(big_blank_durations), dur_ptr,
             int(blank), float(fastemit_lambda), float(clamp), float(sigma), _ptr(workspace), workspace.numel(),
             _stream(acts.device),
         )  # fmt: skip

@@ -1,0 +1,179 @@
+"""Riders of the lattice launch: given the gradient buffer, a forward call zero-fills padded cells of it while the
+lattice recursion runs, as far as it gets, and the backward call with padding_zeroed = 2 skips what was done.
+Whatever the riders managed (nothing on a small problem whose lattice ends before they start, everything beside a
+long TDT lattice), forward + backward must leave exactly what the plain calls leave, the forward call must touch
+padded cells only, and a workspace full of junk must not change any of it."""
+
+import numpy as np
+import pytest
+import torch
+
+from speech_amd import MultiblankRNNTLossNumba, RNNTLossNumba, TDTLossNumba, _native, synthetic
+from speech_amd.rnnt_loss import rnnt, rnnt_pytorch
+
+from gpu_utils import DEV
+
+pytestmark = pytest.mark.gpu
+
+DURATIONS = [0, 1, 2, 3]
+BIG_BLANKS = [2, 4]
+
+
+def make(seed, B, T, U, V, dtype, full=False):
+    rng = np.random.RandomState(seed)
+    acts = torch.tensor(rng.randn(B, T, U, V), dtype=torch.float32).to(dtype).to(DEV)
+    labels = torch.tensor(rng.randint(0, max(V - 6, 1), size=(B, U - 1)), dtype=torch.int64, device=DEV)
+    al, ll = rng.randint(1, T + 1, size=B), rng.randint(0, U, size=B)
+    al[0], ll[-1] = T, U - 1
+    if full:
+        al[:], ll[:] = T, U - 1
+    return acts, labels, torch.tensor(al, device=DEV), torch.tensor(ll, device=DEV)
+
+
+def run(kind, acts, labels, al, ll, prefill, ws=None, scale=None):
+    """(costs, grads, buffer as the forward call left it) through the function-level seam."""
+    B, T, U, V = acts.shape
+    D = {"rnnt": 0, "tdt": len(DURATIONS), "multiblank": len(BIG_BLANKS)}[kind]
+    ws = rnnt.new_workspace(acts, D) if ws is None else ws
+    costs = torch.empty(B, dtype=torch.float32, device=DEV)
+    grads = torch.full_like(acts, float("nan"))
+    pre = grads if prefill else None
+    mode = 2 if prefill else 0
+    if kind == "rnnt":
+        rnnt.rnnt_forward(acts, labels, al, ll, costs, V - 1, 0.01, True, ws, pre)
+        after_forward = grads.clone()
+        rnnt.rnnt_backward(acts, labels, al, ll, grads, scale, V - 1, 0.01, 0.0, ws, padding_zeroed=mode)
+    elif kind == "tdt":
+        rnnt.tdt_forward(acts, labels, al, ll, costs, V - D - 1, DURATIONS, 0.0, 0.05, False, True, ws, pre)
+        after_forward = grads.clone()
+        rnnt.tdt_backward(acts, labels, al, ll, grads, scale, V - D - 1, DURATIONS, 0.0, 0.0, 0.05, False, ws,
+                          padding_zeroed=mode)  # fmt: skip
+    else:
+        rnnt.multiblank_forward(acts, labels, al, ll, costs, V - 1, BIG_BLANKS, 0.0, 0.05, True, ws, pre)
+        after_forward = grads.clone()
+        rnnt.multiblank_backward(acts, labels, al, ll, grads, scale, V - 1, BIG_BLANKS, 0.0, 0.0, 0.05, ws,
+                                 padding_zeroed=mode)  # fmt: skip
+    torch.cuda.synchronize()
+    return costs, grads, after_forward
+
+
+def check_forward_touched_padding_only(after_forward, al, ll):
+    touched = ~torch.isnan(after_forward.float())
+    assert torch.all(after_forward[touched] == 0)
+    for b in range(after_forward.shape[0]):
+        assert not touched[b, : int(al[b]), : int(ll[b]) + 1].any(), "a rider wrote into a valid cell"
+
+
+# V: rows of one vector up to rows that take a workgroup of 1024 threads (one row per item), odd and even starts
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("V", [29, 257, 1025, 4100, 16385])
+@pytest.mark.parametrize("kind", ["rnnt", "tdt", "multiblank"])
+def test_prefilled_gradient_equals_the_plain_gradient(kind, V, dtype):
+    B, T, U = 3, 21, 11  # U is no multiple of the eight rows of an item
+    acts, labels, al, ll = make(V, B, T, U, V, dtype)
+    scale = torch.tensor([0.5, 1.0, 2.0], device=DEV)
+    c0, g0, _ = run(kind, acts, labels, al, ll, False, scale=scale)
+    c1, g1, after_forward = run(kind, acts, labels, al, ll, True, scale=scale)
+    assert torch.isfinite(g0.float()).all()
+    assert torch.equal(c0, c1) and torch.equal(g0, g1)
+    check_forward_touched_padding_only(after_forward, al, ll)
+
+
+@pytest.mark.parametrize("kind", ["rnnt", "tdt", "multiblank"])
+def test_riders_fill_padding_beside_a_long_lattice(kind):
+    """A lattice of several hundred anti-diagonals gives the riders time: they must have filled some padding, only
+    padding, and the result must not change."""
+    B, T, U, V = 4, 300, 40, 257 if kind != "tdt" else 257 + len(DURATIONS)
+    acts, labels, al, ll = make(7, B, T, U, V, torch.float32)
+    al[1], al[2] = 40, 150  # one long utterance keeps the lattice going while the short ones leave padding
+    c0, g0, _ = run(kind, acts, labels, al, ll, False)
+    c1, g1, after_forward = run(kind, acts, labels, al, ll, True)
+    assert torch.equal(c0, c1) and torch.equal(g0, g1)
+    check_forward_touched_padding_only(after_forward, al, ll)
+    assert (~torch.isnan(after_forward)).any(), "the riders filled nothing beside a lattice of 340 anti-diagonals"
+
+
+@pytest.mark.parametrize("kind", ["rnnt", "tdt", "multiblank"])
+@pytest.mark.parametrize("junk", ["nan", "ff", "zero"])
+def test_junk_in_the_workspace_does_not_reach_the_result(kind, junk):
+    B, T, U, V = 3, 60, 13, 300
+    acts, labels, al, ll = make(11, B, T, U, V, torch.float32)
+    c0, g0, _ = run(kind, acts, labels, al, ll, False)
+    D = {"rnnt": 0, "tdt": len(DURATIONS), "multiblank": len(BIG_BLANKS)}[kind]
+    ws = rnnt.new_workspace(acts, D)
+    if junk == "nan":
+        ws.view(torch.float32)[: ws.numel() // 4] = float("nan")
+    elif junk == "ff":
+        ws.fill_(255)
+    else:
+        ws.zero_()
+    c1, g1, after_forward = run(kind, acts, labels, al, ll, True, ws=ws)
+    assert torch.equal(c0, c1) and torch.equal(g0, g1)
+    check_forward_touched_padding_only(after_forward, al, ll)
+    # the same workspace again: what the first call left (its riders' words, its epoch) is not mistaken for news
+    c2, g2, after_forward = run(kind, acts, labels, al, ll, True, ws=ws)
+    assert torch.equal(c0, c2) and torch.equal(g0, g2)
+    check_forward_touched_padding_only(after_forward, al, ll)
+
+
+def test_no_padding_and_batches_too_large_for_riders():
+    # nothing to fill
+    acts, labels, al, ll = make(3, 2, 30, 9, 257, torch.float32, full=True)
+    c0, g0, _ = run("rnnt", acts, labels, al, ll, False)
+    c1, g1, after_forward = run("rnnt", acts, labels, al, ll, True)
+    assert torch.equal(c0, c1) and torch.equal(g0, g1) and torch.isnan(after_forward).all()
+    # more lattice workgroups than the record has room for: no riders, the record is cleared, same result
+    acts, labels, al, ll = make(4, 150, 6, 5, 40, torch.float32)
+    c0, g0, _ = run("rnnt", acts, labels, al, ll, False)
+    c1, g1, after_forward = run("rnnt", acts, labels, al, ll, True)
+    assert torch.equal(c0, c1) and torch.equal(g0, g1) and torch.isnan(after_forward).all()
+
+
+def test_invalid_padding_mode_and_prefill_buffer():
+    acts, labels, al, ll = make(5, 2, 8, 5, 40, torch.float32)
+    ws = rnnt.new_workspace(acts)
+    costs = torch.empty(2, dtype=torch.float32, device=DEV)
+    grads = torch.empty_like(acts)
+    rnnt.rnnt_forward(acts, labels, al, ll, costs, 39, 0.0, True, ws)
+    with pytest.raises(RuntimeError):
+        rnnt.rnnt_backward(acts, labels, al, ll, grads, None, 39, 0.0, 0.0, ws, padding_zeroed=3)
+    with pytest.raises(ValueError):
+        rnnt.rnnt_forward(acts, labels, al, ll, costs, 39, 0.0, True, ws, grads[:, :-1])
+    with pytest.raises(ValueError):
+        rnnt.rnnt_forward(acts, labels, al, ll, costs, 39, 0.0, True, ws, grads.to(torch.bfloat16))
+
+
+@pytest.mark.parametrize("kind", ["rnnt", "tdt", "multiblank"])
+def test_module_with_and_without_prefill(kind, monkeypatch):
+    """The modules hand the lattice launch their gradient buffer by default on problems this size; switched off they
+    must return the same costs and gradients, also from a logits view that starts off a 16-byte boundary, and a
+    second backward call through a retained graph must not reuse the prefilled buffer."""
+    index = {"rnnt": 1, "tdt": 3, "multiblank": 5}[kind]
+    cfg, acts, labels, al, ll = synthetic.make_inputs(index, device=DEV, generate_on_device=True)
+    B = 4  # a slice of the benchmark batch: ragged lengths, a lattice of several hundred anti-diagonals
+    flat = torch.empty(acts[:B].numel() + 1, dtype=acts.dtype, device=DEV)
+    view = flat[1:].view(acts[:B].shape)
+    view.copy_(acts[:B])
+    labels, al, ll = labels[:B].contiguous(), al[:B].clone(), ll[:B].clone()
+    al[0], ll[B - 1] = acts.shape[1], acts.shape[2] - 1  # (the modules insist on one utterance of full length each way)
+    if kind == "rnnt":
+        loss = RNNTLossNumba(blank=cfg.blank, reduction="none", fastemit_lambda=0.001)
+    elif kind == "tdt":
+        loss = TDTLossNumba(blank=cfg.blank, durations=cfg.durations, reduction="none", sigma=cfg.sigma)
+    else:
+        loss = MultiblankRNNTLossNumba(blank=cfg.blank, big_blank_durations=cfg.big_blank_durations, reduction="none",
+                                       sigma=cfg.sigma)  # fmt: skip
+    out = {}
+    for mode in ("0", "1"):
+        monkeypatch.setattr(rnnt_pytorch, "_PREFILL_ENV", mode)
+        a = view.detach().requires_grad_(True)
+        costs = loss(a, labels, al, ll)
+        (g1,) = torch.autograd.grad(costs.sum(), a, retain_graph=True)
+        (g2,) = torch.autograd.grad((2.0 * costs).sum(), a)
+        torch.cuda.synchronize()
+        out[mode] = (costs.detach().clone(), g1.clone(), g2.clone())
+    assert torch.equal(out["0"][0], out["1"][0])
+    assert torch.equal(out["0"][1], out["1"][1]) and torch.equal(out["0"][2], out["1"][2])
+    assert torch.isfinite(out["1"][1]).all() and out["1"][1].abs().sum() > 0
+    for b in range(B):
+        assert torch.all(out["1"][1][b, int(al[b]) :] == 0) and torch.all(out["1"][1][b, :, int(ll[b]) + 1 :] == 0)

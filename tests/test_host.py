@@ -44,8 +44,8 @@ def test_workspace_size_and_invalid_dimensions(built_lib):
 
 def test_null_and_bad_arguments_return_invalid_value_without_touching_the_gpu(built_lib):
     # every check happens on the host before any HIP call
-    assert built_lib.mi_rnnt_forward(None, 0, None, None, None, None, 1, 2, 3, 4, 0, 0.0, 0, None, 0, None) == 1
-    assert built_lib.mi_tdt_forward(None, 0, None, None, None, None, 1, 2, 3, 4, 2, None, 0, 0.0, 0.0, 0, 0, None, 0, None) == 1
+    assert built_lib.mi_rnnt_forward(None, 0, None, None, None, None, 1, 2, 3, 4, 0, 0.0, 0, None, None, 0, None) == 1
+    assert built_lib.mi_tdt_forward(None, 0, None, None, None, None, 1, 2, 3, 4, 2, None, 0, 0.0, 0.0, 0, 0, None, None, 0, None) == 1
     assert built_lib.mi_transducer_length_maxima(None, None, 1, None, None) == 1
 
 
