@@ -363,7 +363,8 @@ int mi_transducer_length_maxima(const int64_t* act_lens, const int64_t* label_le
 
 /* ---- diagnostics ------------------------------------------------------------------------
  * Everything from here to the end of this header (mi_transducer_profile_*, mi_transducer_describe_plan,
- * mi_transducer_copy_probe, mi_transducer_set_lattice_mode, mi_transducer_scale_segment) binds NO interface of the reference: these are aids for benchmarks, profiles and tests
+ * mi_transducer_copy_probe, mi_transducer_set_lattice_mode, mi_transducer_scale_segment,
+ * mi_transducer_prefill_record) binds NO interface of the reference: these are aids for benchmarks, profiles and tests
  * of this library, and a drop-in user of the loss never calls them.
  *
  * Per-kernel timing of the launches a harness itself makes: after
@@ -412,6 +413,14 @@ int mi_transducer_set_lattice_mode(int mode);
  * Host arithmetic only.  For tests that must know which of the two recursions produced a result. */
 int mi_transducer_scale_segment(int B, int T, int U, int D, size_t* offset_bytes, int* ints_per_utterance,
                                 int* format_word);
+
+/* Where a workspace of this shape keeps the record of what the riders of the last forward call with prefill_grads
+ * zero-filled: `*words` int32 starting at byte `*offset_bytes`.  Rows of row_bytes bytes go `*rows_per_item` to an
+ * item (the last item of a frame may be shorter), items are numbered in memory order over (b, t, item of the frame),
+ * and item i has had its padded rows filled iff  i / *words < record[i % *words].  Host arithmetic only.  For
+ * benchmarks that report how many bytes moved from the gradient pass into the lattice launch, and for tests. */
+int mi_transducer_prefill_record(int B, int T, int U, int D, size_t row_bytes, size_t* offset_bytes, int* words,
+                                 int* rows_per_item);
 
 #ifdef __cplusplus
 }

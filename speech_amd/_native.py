@@ -148,6 +148,7 @@ _SIGNATURES = {
     "mi_transducer_copy_probe": [_vp, _vp, _c_size_t, _vp],
     "mi_transducer_set_lattice_mode": [_c_int],
     "mi_transducer_scale_segment": [_c_int, _c_int, _c_int, _c_int, _vp, _vp, _vp],
+    "mi_transducer_prefill_record": [_c_int, _c_int, _c_int, _c_int, _c_size_t, _vp, _vp, _vp],
 }  # fmt: skip
 
 EXPORTED_SYMBOLS = tuple(_SIGNATURES)

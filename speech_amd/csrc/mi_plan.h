@@ -33,8 +33,9 @@ constexpr int kScaleMaxBlocks = 2048;  // exponent tracks the scaled lattice ker
 // An item is 2^prefill_log_rows rows of one frame (b, t), items are numbered in memory order, and item i is the
 // (i / kFillMaxRiders)-th item of virtual rider i % kFillMaxRiders: it is done iff  i / kFillMaxRiders <
 // progress[i % kFillMaxRiders].  A launch has a power of two of real riders, each standing for the virtual riders
-// congruent to it.  The epoch changes with every launch: what an earlier call left in the first two blocks is not
-// mistaken for this call's.
+// congruent to it.  The first two blocks are cleared by pass 1 and stamped with an epoch that changes with every
+// call, so what an earlier call left there is not mistaken for this call's -- also not in a captured graph, where
+// the epoch is frozen.
 constexpr int kFillMaxLattice = 256;
 constexpr int kFillMaxRiders = 4096;
 constexpr int kFillProgress = 2 * kFillMaxLattice;

@@ -399,6 +399,17 @@ int mi_transducer_scale_segment(int B, int T, int U, int D, size_t* offset_bytes
   return MI_TRANSDUCER_SUCCESS;
 }
 
+int mi_transducer_prefill_record(int B, int T, int U, int D, size_t row_bytes, size_t* offset_bytes, int* words,
+                                 int* rows_per_item) {
+  Layout L;
+  if (!offset_bytes || !words || !rows_per_item || row_bytes == 0 || !make_layout(B, T, U, D, &L))
+    return MI_TRANSDUCER_INVALID_VALUE;
+  *offset_bytes = L.off_fill + (size_t)kFillProgress * sizeof(int);
+  *words = kFillMaxRiders;
+  *rows_per_item = 1 << prefill_log_rows(row_bytes);
+  return MI_TRANSDUCER_SUCCESS;
+}
+
 int mi_transducer_set_lattice_mode(int mode) {
   if (mode < 0 || mode > 2) return MI_TRANSDUCER_INVALID_VALUE;
   g_lattice_mode.store(mode, std::memory_order_relaxed);

@@ -297,6 +297,25 @@ def lattice_diagnostics(workspace, B, T, U):
     return seg[:, 2:4].clone()
 
 
+def prefilled_cells(workspace, act_lens, label_lens, B, T, U, row_elems, elem_bytes, num_durations=0):
+    """bool[B, T, U]: the padded cells whose gradient rows the riders of the last forward call with prefill_grads
+    zero-filled, read from the record in `workspace`.  row_elems = V + D of the gradient rows."""
+    off, words, rows = ctypes.c_size_t(0), ctypes.c_int(0), ctypes.c_int(0)
+    status = _native.lib().mi_transducer_prefill_record(
+        B, T, U, num_durations, int(row_elems) * int(elem_bytes), ctypes.byref(off), ctypes.byref(words), ctypes.byref(rows)
+    )
+    _native.check_status(status, "prefill_record")
+    record = workspace[off.value : off.value + 4 * words.value].view(torch.int32).to(torch.int64)
+    dev = workspace.device
+    per_frame = (U + rows.value - 1) // rows.value
+    u = torch.arange(U, device=dev)
+    item = torch.arange(B * T, device=dev).view(B, T, 1) * per_frame + (u // rows.value).view(1, 1, U)
+    done = torch.div(item, words.value, rounding_mode="floor") < record[item % words.value]
+    t = torch.arange(T, device=dev).view(1, T, 1)
+    padded = (t >= act_lens.view(B, 1, 1)) | (u.view(1, 1, U) > label_lens.view(B, 1, 1))
+    return done & padded
+
+
 def _require_cpu_f32(t, what):
     if t.is_cuda or t.dtype != torch.float32 or not t.is_contiguous():
         raise ValueError(f"{what} must be a contiguous float32 CPU tensor")

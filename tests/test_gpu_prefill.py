@@ -57,11 +57,15 @@ def run(kind, acts, labels, al, ll, prefill, ws=None, scale=None):
     return costs, grads, after_forward
 
 
-def check_forward_touched_padding_only(after_forward, al, ll):
+def check_forward_touched_padding_only(after_forward, al, ll, ws=None, D=0):
     touched = ~torch.isnan(after_forward.float())
     assert torch.all(after_forward[touched] == 0)
     for b in range(after_forward.shape[0]):
         assert not touched[b, : int(al[b]), : int(ll[b]) + 1].any(), "a rider wrote into a valid cell"
+    if ws is not None:  # the record names exactly the cells that were filled (whole rows)
+        B, T, U, V = after_forward.shape
+        said = rnnt.prefilled_cells(ws, al, ll, B, T, U, V, after_forward.element_size(), D)
+        assert torch.equal(said, touched.all(dim=-1)) and torch.equal(said, touched.any(dim=-1))
 
 
 # V: rows of one vector up to rows that take a workgroup of 1024 threads (one row per item), odd and even starts
@@ -87,9 +91,11 @@ def test_riders_fill_padding_beside_a_long_lattice(kind):
     acts, labels, al, ll = make(7, B, T, U, V, torch.float32)
     al[1], al[2] = 40, 150  # one long utterance keeps the lattice going while the short ones leave padding
     c0, g0, _ = run(kind, acts, labels, al, ll, False)
-    c1, g1, after_forward = run(kind, acts, labels, al, ll, True)
+    D = {"rnnt": 0, "tdt": len(DURATIONS), "multiblank": len(BIG_BLANKS)}[kind]
+    ws = rnnt.new_workspace(acts, D)
+    c1, g1, after_forward = run(kind, acts, labels, al, ll, True, ws=ws)
     assert torch.equal(c0, c1) and torch.equal(g0, g1)
-    check_forward_touched_padding_only(after_forward, al, ll)
+    check_forward_touched_padding_only(after_forward, al, ll, ws, D)
     assert (~torch.isnan(after_forward)).any(), "the riders filled nothing beside a lattice of 340 anti-diagonals"
 
 
@@ -109,7 +115,7 @@ def test_junk_in_the_workspace_does_not_reach_the_result(kind, junk):
         ws.zero_()
     c1, g1, after_forward = run(kind, acts, labels, al, ll, True, ws=ws)
     assert torch.equal(c0, c1) and torch.equal(g0, g1)
-    check_forward_touched_padding_only(after_forward, al, ll)
+    check_forward_touched_padding_only(after_forward, al, ll, ws, D)
     # the same workspace again: what the first call left (its riders' words, its epoch) is not mistaken for news
     c2, g2, after_forward = run(kind, acts, labels, al, ll, True, ws=ws)
     assert torch.equal(c0, c2) and torch.equal(g0, g2)
@@ -177,3 +183,47 @@ def test_module_with_and_without_prefill(kind, monkeypatch):
     assert torch.isfinite(out["1"][1]).all() and out["1"][1].abs().sum() > 0
     for b in range(B):
         assert torch.all(out["1"][1][b, int(al[b]) :] == 0) and torch.all(out["1"][1][b, :, int(ll[b]) + 1 :] == 0)
+
+
+@pytest.mark.parametrize("kind", ["rnnt", "tdt", "multiblank"])
+def test_replayed_from_a_graph(kind):
+    """Captured once and replayed, the launch's epoch is the same every time: the riders must still tell this replay's
+    lattice from the last one's (they did nothing on replays when they could not), and every replay must give the
+    eager result."""
+    B, T, U, V = 4, 300, 40, 257 if kind != "tdt" else 257 + len(DURATIONS)
+    D = {"rnnt": 0, "tdt": len(DURATIONS), "multiblank": len(BIG_BLANKS)}[kind]
+    acts, labels, al, ll = make(9, B, T, U, V, torch.float32)
+    al[1], al[2] = 40, 150
+    c0, g0, _ = run(kind, acts, labels, al, ll, False)
+    ws = rnnt.new_workspace(acts, D)
+    costs = torch.empty(B, dtype=torch.float32, device=DEV)
+    grads = torch.full_like(acts, float("nan"))
+
+    def step():
+        if kind == "rnnt":
+            rnnt.rnnt_forward(acts, labels, al, ll, costs, V - 1, 0.01, True, ws, grads)
+            rnnt.rnnt_backward(acts, labels, al, ll, grads, None, V - 1, 0.01, 0.0, ws, padding_zeroed=2)
+        elif kind == "tdt":
+            rnnt.tdt_forward(acts, labels, al, ll, costs, V - D - 1, DURATIONS, 0.0, 0.05, False, True, ws, grads)
+            rnnt.tdt_backward(acts, labels, al, ll, grads, None, V - D - 1, DURATIONS, 0.0, 0.0, 0.05, False, ws,
+                              padding_zeroed=2)  # fmt: skip
+        else:
+            rnnt.multiblank_forward(acts, labels, al, ll, costs, V - 1, BIG_BLANKS, 0.0, 0.05, True, ws, grads)
+            rnnt.multiblank_backward(acts, labels, al, ll, grads, None, V - 1, BIG_BLANKS, 0.0, 0.0, 0.05, ws,
+                                     padding_zeroed=2)  # fmt: skip
+
+    step()
+    torch.cuda.synchronize()
+    assert torch.equal(g0, grads)
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        step()
+    for replay in range(4):
+        grads.fill_(float("nan"))  # eager work between the replays
+        costs.fill_(float("nan"))
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(c0, costs) and torch.equal(g0, grads), f"replay {replay}"
+        said = rnnt.prefilled_cells(ws, al, ll, B, T, U, V, 4, D)
+        assert said.any(), f"the riders did nothing on replay {replay}"
