@@ -364,7 +364,7 @@ int mi_transducer_length_maxima(const int64_t* act_lens, const int64_t* label_le
 /* ---- diagnostics ------------------------------------------------------------------------
  * Everything from here to the end of this header (mi_transducer_profile_*, mi_transducer_describe_plan,
  * mi_transducer_copy_probe, mi_transducer_set_lattice_mode, mi_transducer_scale_segment,
- * mi_transducer_prefill_record) binds NO interface of the reference: these are aids for benchmarks, profiles and tests
+ * mi_transducer_prefill_record, mi_transducer_set_prefill_min_bytes) binds NO interface of the reference: these are aids for benchmarks, profiles and tests
  * of this library, and a drop-in user of the loss never calls them.
  *
  * Per-kernel timing of the launches a harness itself makes: after
@@ -421,6 +421,11 @@ int mi_transducer_scale_segment(int B, int T, int U, int D, size_t* offset_bytes
  * benchmarks that report how many bytes moved from the gradient pass into the lattice launch, and for tests. */
 int mi_transducer_prefill_record(int B, int T, int U, int D, size_t row_bytes, size_t* offset_bytes, int* words,
                                  int* rows_per_item);
+
+/* A forward call given prefill_grads launches riders only if the gradient tensor has at least this many bytes
+ * (process-wide; 32 MiB unless set): below that a step is bound by its launches.  Tests set it to 0 so that small
+ * shapes run the riders too. */
+int mi_transducer_set_prefill_min_bytes(size_t bytes);
 
 #ifdef __cplusplus
 }

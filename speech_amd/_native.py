@@ -149,6 +149,7 @@ _SIGNATURES = {
     "mi_transducer_set_lattice_mode": [_c_int],
     "mi_transducer_scale_segment": [_c_int, _c_int, _c_int, _c_int, _vp, _vp, _vp],
     "mi_transducer_prefill_record": [_c_int, _c_int, _c_int, _c_int, _c_size_t, _vp, _vp, _vp],
+    "mi_transducer_set_prefill_min_bytes": [_c_size_t],
 }  # fmt: skip
 
 EXPORTED_SYMBOLS = tuple(_SIGNATURES)

@@ -410,6 +410,11 @@ int mi_transducer_prefill_record(int B, int T, int U, int D, size_t row_bytes, s
   return MI_TRANSDUCER_SUCCESS;
 }
 
+int mi_transducer_set_prefill_min_bytes(size_t bytes) {
+  g_prefill_min_bytes.store(bytes, std::memory_order_relaxed);
+  return MI_TRANSDUCER_SUCCESS;
+}
+
 int mi_transducer_set_lattice_mode(int mode) {
   if (mode < 0 || mode > 2) return MI_TRANSDUCER_INVALID_VALUE;
   g_lattice_mode.store(mode, std::memory_order_relaxed);

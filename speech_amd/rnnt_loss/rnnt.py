@@ -297,6 +297,11 @@ def lattice_diagnostics(workspace, B, T, U):
     return seg[:, 2:4].clone()
 
 
+def set_prefill_min_bytes(nbytes):
+    """Gradient tensors below this size get no riders in their lattice launch (process-wide; 32 MiB unless set)."""
+    _native.check_status(_native.lib().mi_transducer_set_prefill_min_bytes(int(nbytes)), "set_prefill_min_bytes")
+
+
 def prefilled_cells(workspace, act_lens, label_lens, B, T, U, row_elems, elem_bytes, num_durations=0):
     """bool[B, T, U]: the padded cells whose gradient rows the riders of the last forward call with prefill_grads
     zero-filled, read from the record in `workspace`.  row_elems = V + D of the gradient rows."""

@@ -15,6 +15,15 @@ from gpu_utils import DEV
 
 pytestmark = pytest.mark.gpu
 
+
+
+@pytest.fixture(autouse=True)
+def riders_for_every_size():
+    rnnt.set_prefill_min_bytes(0)  # the shapes here are far below the size from which a forward call takes riders
+    yield
+    rnnt.set_prefill_min_bytes(32 << 20)
+
+
 DURATIONS = [0, 1, 2, 3]
 BIG_BLANKS = [2, 4]
 
@@ -227,3 +236,13 @@ def test_replayed_from_a_graph(kind):
         assert torch.equal(c0, costs) and torch.equal(g0, grads), f"replay {replay}"
         said = rnnt.prefilled_cells(ws, al, ll, B, T, U, V, 4, D)
         assert said.any(), f"the riders did nothing on replay {replay}"
+
+
+def test_small_gradients_get_no_riders():
+    B, T, U, V = 4, 300, 40, 257
+    acts, labels, al, ll = make(7, B, T, U, V, torch.float32)
+    al[1], al[2] = 40, 150
+    rnnt.set_prefill_min_bytes(acts.numel() * 4 + 1)
+    c0, g0, _ = run("rnnt", acts, labels, al, ll, False)
+    c1, g1, after_forward = run("rnnt", acts, labels, al, ll, True)
+    assert torch.equal(c0, c1) and torch.equal(g0, g1) and torch.isnan(after_forward).all()
