@@ -43,7 +43,7 @@ HBM_PEAK_GBPS = 8000.0  # MI355X HBM3E, published peak
 MEASURED_TRAFFIC_BYTES = {
     # profiles/transducer_kernels_cfg2_hbm_traffic.md: fetch 1.6485 GB + write 2.6671 GB (the lattice launch, whose
     # riders zero-fill part of the padding, writes another 0.33 GB)
-    ("cfg2_rnnt_B16_T375_U121_V1025_f32", False): int((804936 * 2.0 + 2604584) * 1024),
+    "cfg2_rnnt_B16_T375_U121_V1025_f32": int((804936 * 2.0 + 2604584) * 1024),
 }
 
 
@@ -514,16 +514,13 @@ def main():
 
     grad_ms, grad_n = kernels["gradient_pass"]
     grad_avg_s = grad_ms * 1e-3 / max(grad_n, 1)
-    # with the padding zero-filled by its own kernel during forward, the gradient pass reads and
-    # writes the valid rows only
-    overlap = rnnt_pytorch.OVERLAP_PADDING and not logprobs
     if logprobs:  # the op's backward always streams the coefficient records of its own cell kernel
         plan["lattice"], plan["cells"] = "none", "logprobs_export_kernel + logprobs_cell_kernel"
         plan["gradient"] = plan["gradient"].replace("fused>", "coef>")
-    grad_bytes = nbytes["grad_valid"] if overlap else nbytes["grad_stream"]
+    grad_bytes = nbytes["grad_stream"]
     # the riders of the lattice launch zero-fill part of the padding while the recursion runs; those bytes are the
     # lattice launch's, not the gradient pass's
-    riders_bytes = 0 if (logprobs or overlap) else riders_filled_bytes(torch, cfg, acts.detach(), labels, act_lens, label_lens)
+    riders_bytes = 0 if logprobs else riders_filled_bytes(torch, cfg, acts.detach(), labels, act_lens, label_lens)
     grad_bytes -= riders_bytes
     achieved = grad_bytes / grad_avg_s / 1e9
     result = {
@@ -563,10 +560,9 @@ def main():
             "peak": HBM_PEAK_GBPS,
             "unit": "GB/s",
             "frac": achieved / HBM_PEAK_GBPS,
-            "traffic": None if logprobs else MEASURED_TRAFFIC_BYTES.get((cfg.name, overlap)),
+            "traffic": None if logprobs else MEASURED_TRAFFIC_BYTES.get(cfg.name),
             "algorithmic_bytes_per_launch": grad_bytes,
-            "padding_zero_filled_by": ("zero_padding_kernel (second stream, during forward)" if overlap else
-                                       "this kernel, less what the riders of the lattice launch did"),
+            "padding_zero_filled_by": "this kernel, less what the riders of the lattice launch did",
             "riders_filled_bytes": riders_bytes,
             "avg_launch_ms": grad_avg_s * 1e3,
             "launches": grad_n,

@@ -39,13 +39,6 @@ __all__ = [
 ]  # fmt: skip
 
 
-# Optional (MI_TRANSDUCER_OVERLAP=1): when the gradient will be needed, forward allocates it and,
-# once the denominators are done, zero-fills its padded cells on a second stream while the lattice
-# recursion runs; backward then writes the valid cells only and joins the two streams.  Off by
-# default: the recursion is a chain of dependent memory round trips, and a fill that saturates HBM
-# beside it stretches every step of the chain, so the measured step time is no better than with
-# backward writing the whole gradient in one pass.
-OVERLAP_PADDING = os.environ.get("MI_TRANSDUCER_OVERLAP", "0") == "1"
 
 # The gradient of padded cells is zeros that depend on the lengths alone.  When the gradient will be needed, forward
 # allocates it and hands it to the lattice launch, whose extra workgroups write those zeros while the recursion runs
@@ -71,20 +64,6 @@ def _aux_stream(device):
         stream = torch.cuda.Stream(device=device)  # default priority
         _aux_streams[device.index] = stream
     return stream
-
-
-def _start_padding_fill(grads, act_lens, label_lens):
-    """Enqueue the zero-fill of the padded cells of grads on the auxiliary stream, ordered after
-    everything enqueued so far on the current stream.  Returns the event recorded after the fill."""
-    main = torch.cuda.current_stream(grads.device)
-    aux = _aux_stream(grads.device)
-    aux.wait_stream(main)
-    with torch.cuda.stream(aux):
-        rnnt.zero_padding(grads, act_lens, label_lens)
-        done = torch.cuda.Event()
-        done.record(aux)
-    grads.record_stream(aux)
-    return done
 
 
 def grads_like(acts):
@@ -305,18 +284,9 @@ class _RNNTNumba(Function):
             batch = acts.size(0)
             costs = torch.empty(batch, device=acts.device, dtype=torch.float32)
             workspace = rnnt.new_workspace(acts)
-            ctx.padding = None
-            ctx.prefilled = None
-            if need_grad and OVERLAP_PADDING:
-                grads = grads_like(acts)
-                rnnt.denominators(acts, labels, act_lens, label_lens, blank, workspace)
-                ctx.padding = (grads, _start_padding_fill(grads, act_lens, label_lens))
-                B, T, U = acts.shape[:3]
-                rnnt.rnnt_lattice(act_lens, label_lens, costs, B, T, U, fastemit_lambda, True, workspace)
-            else:
-                ctx.prefilled = grads_like(acts) if need_grad and _prefill_wanted(acts) else None
-                rnnt.rnnt_forward(acts, labels, act_lens, label_lens, costs, blank, fastemit_lambda, need_grad, workspace,
-                                  ctx.prefilled)
+            ctx.prefilled = grads_like(acts) if need_grad and _prefill_wanted(acts) else None
+            rnnt.rnnt_forward(acts, labels, act_lens, label_lens, costs, blank, fastemit_lambda, need_grad, workspace,
+                              ctx.prefilled)
         except BaseException:
             pending.drain()  # the pinned buffer must outlive the kernel that writes into it
             raise
@@ -339,16 +309,13 @@ class _RNNTNumba(Function):
             rnnt.rnnt_cpu_backward(acts, labels, act_lens, label_lens, grads, scale, blank, fastemit_lambda, clamp,
                                    workspace, 1 if scale.numel() > 1 else 0, mul)  # fmt: skip
             return grads, None, None, None, None, None, None, None
-        prepared, ctx.padding = ctx.padding, None  # the prepared buffer serves the first backward call only
-        prefilled, ctx.prefilled = ctx.prefilled, None
-        grads = prepared[0] if prepared else (prefilled if prefilled is not None else grads_like(acts))
+        prefilled, ctx.prefilled = ctx.prefilled, None  # the prefilled buffer serves the first backward call only
+        grads = prefilled if prefilled is not None else grads_like(acts)
         scale, stride, mul = _grad_scale(grad_output, reduction, acts.size(0), acts.device)
         rnnt.rnnt_backward(
             acts, labels, act_lens, label_lens, grads, scale, blank, fastemit_lambda, clamp, workspace, stride, mul,
-            1 if prepared else (2 if prefilled is not None else 0),
+            2 if prefilled is not None else 0,
         )  # fmt: skip
-        if prepared:
-            torch.cuda.current_stream(acts.device).wait_event(prepared[1])  # join the padding fill
         return grads, None, None, None, None, None, None, None
 
 
@@ -377,24 +344,11 @@ class _TDTNumba(Function):
             workspace = rnnt.new_workspace(acts, len(durations))
             # gpu_rnnt.py:606-607: one host-side draw per call decides between the TDT and the plain RNNT kernels
             use_plain_rnnt = random.uniform(0, 1) < omega
-            ctx.padding = None
-            ctx.prefilled = None
-            if need_grad and OVERLAP_PADDING:
-                grads = grads_like(acts)
-                D = len(durations)
-                rnnt.denominators(acts, labels, act_lens, label_lens, blank, workspace, D)
-                ctx.padding = (grads, _start_padding_fill(grads, act_lens, label_lens))
-                B, T, U = acts.shape[:3]
-                if use_plain_rnnt:
-                    rnnt.rnnt_lattice(act_lens, label_lens, costs, B, T, U, fastemit_lambda, True, workspace, D)
-                else:
-                    rnnt.tdt_lattice(act_lens, label_lens, costs, B, T, U, durations, fastemit_lambda, sigma, True, workspace)
-            else:
-                ctx.prefilled = grads_like(acts) if need_grad and _prefill_wanted(acts) else None
-                rnnt.tdt_forward(
-                    acts, labels, act_lens, label_lens, costs, blank, durations, fastemit_lambda, sigma, use_plain_rnnt,
-                    need_grad, workspace, ctx.prefilled,
-                )  # fmt: skip
+            ctx.prefilled = grads_like(acts) if need_grad and _prefill_wanted(acts) else None
+            rnnt.tdt_forward(
+                acts, labels, act_lens, label_lens, costs, blank, durations, fastemit_lambda, sigma, use_plain_rnnt,
+                need_grad, workspace, ctx.prefilled,
+            )  # fmt: skip
         except BaseException:
             pending.drain()  # the pinned buffer must outlive the kernel that writes into it
             raise
@@ -413,16 +367,13 @@ class _TDTNumba(Function):
     def backward(ctx, grad_output):
         acts, labels, act_lens, label_lens, workspace = ctx.saved_tensors
         blank, durations, reduction, fastemit_lambda, clamp, sigma, use_plain_rnnt = ctx.params
-        prepared, ctx.padding = ctx.padding, None
-        prefilled, ctx.prefilled = ctx.prefilled, None
-        grads = prepared[0] if prepared else (prefilled if prefilled is not None else grads_like(acts))
+        prefilled, ctx.prefilled = ctx.prefilled, None  # (serves the first backward call only)
+        grads = prefilled if prefilled is not None else grads_like(acts)
         scale, stride, mul = _grad_scale(grad_output, reduction, acts.size(0), acts.device)
         rnnt.tdt_backward(
             acts, labels, act_lens, label_lens, grads, scale, blank, durations, fastemit_lambda, clamp, sigma,
-            use_plain_rnnt, workspace, stride, mul, 1 if prepared else (2 if prefilled is not None else 0),
+            use_plain_rnnt, workspace, stride, mul, 2 if prefilled is not None else 0,
         )  # fmt: skip
-        if prepared:
-            torch.cuda.current_stream(acts.device).wait_event(prepared[1])
         return grads, None, None, None, None, None, None, None, None, None, None
 
 
