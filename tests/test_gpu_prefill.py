@@ -246,3 +246,36 @@ def test_small_gradients_get_no_riders():
     c0, g0, _ = run("rnnt", acts, labels, al, ll, False)
     c1, g1, after_forward = run("rnnt", acts, labels, al, ll, True)
     assert torch.equal(c0, c1) and torch.equal(g0, g1) and torch.isnan(after_forward).all()
+
+
+@pytest.mark.parametrize("omega", [0.0, 1.0])
+def test_function_level_seams_take_riders_by_themselves(omega):
+    """rnnt_loss_gpu / tdt_loss_gpu (the reference's signatures: split token logits and duration log-probs, also its
+    plain-RNNT branch) / combined_tdt_loss_gpu / multiblank_rnnt_loss_gpu hand their gradient buffer to the lattice
+    launch on their own: with the size threshold at 0 and out of reach the results must be the same bits."""
+    B, T, U, V, D = 4, 200, 30, 130, len(DURATIONS)
+    acts, labels, al, ll = make(13, B, T, U, V + D, torch.float32)
+    al[1], al[2] = 30, 90
+    label_acts = acts[..., :V].contiguous()
+    duration_acts = torch.log_softmax(acts[..., V:], dim=-1).contiguous()
+    mb_acts = acts[..., : V + len(BIG_BLANKS)].contiguous()
+    out = {}
+    for threshold in (0, 1 << 40):
+        rnnt.set_prefill_min_bytes(threshold)
+        res = []
+        costs, grads = torch.empty(B, device=DEV), torch.full_like(label_acts, float("nan"))
+        rnnt.rnnt_loss_gpu(label_acts, labels, al, ll, costs, grads, V - 1, 0.01, 0.0)
+        res += [costs, grads]
+        costs, lg, dg = torch.empty(B, device=DEV), torch.full_like(label_acts, float("nan")), torch.full_like(duration_acts, float("nan"))
+        rnnt.tdt_loss_gpu(label_acts, duration_acts, labels, al, ll, costs, lg, dg, V - 1, DURATIONS, 0.0, 0.0, 0, 0.05, omega)
+        res += [costs, lg, dg]
+        costs, grads = torch.empty(B, device=DEV), torch.full_like(acts, float("nan"))
+        rnnt.combined_tdt_loss_gpu(acts, labels, al, ll, costs, grads, V - 1, DURATIONS, 0.0, 0.0, 0, 0.05, omega > 0.5)
+        res += [costs, grads]
+        costs, grads = torch.empty(B, device=DEV), torch.full_like(mb_acts, float("nan"))
+        rnnt.multiblank_rnnt_loss_gpu(mb_acts, labels, al, ll, costs, grads, V + len(BIG_BLANKS) - 1, BIG_BLANKS, 0.0, 0.0, 0, 0.05)
+        res += [costs, grads]
+        torch.cuda.synchronize()
+        out[threshold] = res
+    for a, b in zip(out[0], out[1 << 40]):
+        assert torch.isfinite(a).all() and torch.equal(a, b)
