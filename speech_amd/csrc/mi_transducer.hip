@@ -326,8 +326,12 @@ int mi_multiblank_backward(const void* acts, int act_dtype, const int64_t* label
   if (st) return st;
   const ScaleArg sc = {grad_scale, grad_scale_stride, grad_mul};
   if ((st = run_multiblank_cells(c, sc, fastemit_lambda, clamp, prm))) return st;
-  if ((st = run_grad_stream(c, grads, padding_flags(padding_zeroed), false, sc, fastemit_lambda, clamp))) return st;
-  return run_multiblank_fixup(c, grads, prm);
+  // the workgroup-per-row gradient kernel writes the big blanks' entries itself; behind the other kernels a small
+  // kernel overwrites them
+  const bool folded = grad_block_plan(c, grads).RT != 0;
+  const int flags = padding_flags(padding_zeroed) | (folded ? prm.NB << kFlagBigBlanksShift : 0);
+  if ((st = run_grad_stream(c, grads, flags, false, sc, fastemit_lambda, clamp))) return st;
+  return folded ? MI_TRANSDUCER_SUCCESS : run_multiblank_fixup(c, grads, prm);
 }
 
 int mi_multiblank_loss(const void* acts, int act_dtype, const int64_t* labels, const int64_t* act_lens,
