@@ -208,12 +208,10 @@ int mi_multiblank_loss(const void* acts, int act_dtype, const int64_t* labels, c
  * them and for stage-level tests.  They mirror the reference's separately launched kernels:
  * reduce_max/reduce_exp (utils/cuda_utils/reduce.py:299-362) and compute_alphas/betas_kernel
  * (utils/cuda_utils/gpu_rnnt_kernel.py:73-269, :888-1241).  D = 0 for RNNT; the lattice calls need
- * the D the denominators were run with (it fixes the workspace layout).  With D > 0 the denominators are told which
- * lattice follows: use_plain_rnnt = 0 -> mi_tdt_lattice, != 0 -> mi_rnnt_lattice (the omega branch); the two read
- * the arc log-probs in different arrangements. */
+ * the D the denominators were run with (it fixes the workspace layout). */
 int mi_transducer_denominators(const void* acts, int act_dtype, const int64_t* labels, const int64_t* act_lens,
-                               const int64_t* label_lens, int B, int T, int U, int V, int D, int use_plain_rnnt,
-                               int blank, void* workspace, size_t workspace_bytes, void* stream);
+                               const int64_t* label_lens, int B, int T, int U, int V, int D, int blank,
+                               void* workspace, size_t workspace_bytes, void* stream);
 int mi_rnnt_lattice(const int64_t* act_lens, const int64_t* label_lens, float* costs, int B, int T, int U, int D,
                     float fastemit_lambda, int with_betas, void* workspace, size_t workspace_bytes, void* stream);
 int mi_tdt_lattice(const int64_t* act_lens, const int64_t* label_lens, float* costs, int B, int T, int U, int D,

@@ -21,7 +21,7 @@ CPU_SOURCES = [os.path.join(CSRC_DIR, "mi_cpu.cpp")]
 CPU_ABI_VERSION = 1
 CXX_FLAGS = ["-O3", "-std=c++17", "-fPIC", "-shared", "-fopenmp", "-Wall", "-Wextra"]
 
-ABI_VERSION = 18
+ABI_VERSION = 17
 SUCCESS, INVALID_VALUE, LAUNCH_FAILURE, TOO_LARGE = 0, 1, 2, 3
 STATIC_WORKSPACE_BYTES = 64 << 20
 DTYPE_F32, DTYPE_BF16, DTYPE_F16 = 0, 1, 2
@@ -134,7 +134,7 @@ _SIGNATURES = {
     "mi_transducer_export_lattice": [_vp, _c_size_t, _vp, _vp, _c_int, _c_int, _c_int, _c_int, _vp, _vp, _vp, _vp,
                                      _vp, _vp],
     "mi_transducer_length_maxima": [_vp, _vp, _c_int, _vp, _vp],
-    "mi_transducer_denominators": [_vp, _c_int, _vp, _vp, _vp, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _vp,
+    "mi_transducer_denominators": [_vp, _c_int, _vp, _vp, _vp, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _vp,
                                    _c_size_t, _vp],
     "mi_rnnt_lattice": [_vp, _vp, _vp, _c_int, _c_int, _c_int, _c_int, _c_float, _c_int, _vp, _c_size_t, _vp],
     "mi_tdt_lattice": [_vp, _vp, _vp, _c_int, _c_int, _c_int, _c_int, _vp, _c_float, _c_float, _c_int, _vp, _c_size_t,

@@ -49,20 +49,6 @@ inline int prefill_log_rows(size_t row_bytes) {
   return log_rows;
 }
 
-// Where the arc log-probs of a cell sit in the `arcs` segment: value `plane` (0 blank, 1 label, 2+i duration i or big
-// blank i) of the cell in column u of skewed row n = t + u of utterance b is float number
-//     (b * ND + n) * pitch + u * su + plane * sp.
-// Planes (RNNT, multi-blank, the plain-RNNT branch of TDT): [row][plane][column], so that a lattice wave reads a plane
-// of a row with one vector access per lane.  Records (TDT): [row][column][AP], the A values of a cell together --
-// pass 1 then writes a cell with one store of 28 bytes into one line instead of seven 4-byte stores into seven lines
-// (the skewed planes are written a column at a time, and their lines fill up over many frames), and a lattice thread
-// reads its cell with two 16-byte loads instead of six 4-byte ones.
-struct ArcAddr {
-  int pitch, su, sp;
-};
-inline ArcAddr arc_planes(int A, int Us) { return ArcAddr{A * Us, 1, Us}; }
-inline ArcAddr arc_records(int AP, int Us) { return ArcAddr{Us * AP, AP, 1}; }
-
 // ----------------------------------------------------------------------------------------
 // Workspace layout
 // ----------------------------------------------------------------------------------------
@@ -70,8 +56,7 @@ struct Layout {
   int K;    // lattice cells per lane (1,2,4,8,16)
   int Us;   // pitch of a skewed lattice row = 64*K >= U
   int ND;   // number of anti-diagonals of the padded lattice = T+U-1
-  int A;    // arc values per cell: blank, label, D duration log-probs
-  int AP;   // floats per cell record when the arc values of a cell are kept together (A rounded up to a multiple of 4)
+  int A;    // arc planes per diagonal row: blank, label, D duration log-probs
   int CS;   // floats per cell in the coefficient buffer
   int SG;   // ints per utterance in the scale segment: kScaleHeader, then {alpha, beta} exponent per 8 diagonals
   size_t off_denom, off_arcs, off_alphas, off_betas, off_ll, off_coef, off_scale, off_fill, total;
@@ -88,13 +73,12 @@ inline bool make_layout(int B, int T, int U, int D, Layout* L) {
   L->Us = 64 * K;
   L->ND = T + U - 1;
   L->A = 2 + D;
-  L->AP = (L->A + 3) & ~3;
   L->CS = kCoefBase + ((D + 3) & ~3);
   const size_t cells = (size_t)B * T * U;
   const size_t skew = (size_t)B * L->ND * L->Us;
   size_t off = 0;
   L->off_denom = off;  off = align256(off + cells * sizeof(float));
-  L->off_arcs = off;   off = align256(off + skew * (D > 0 ? L->AP : L->A) * sizeof(float));
+  L->off_arcs = off;   off = align256(off + skew * L->A * sizeof(float));
   L->off_alphas = off; off = align256(off + skew * sizeof(double));
   L->off_betas = off;  off = align256(off + skew * sizeof(double));
   L->off_ll = off;     off = align256(off + (size_t)B * 2 * sizeof(double));

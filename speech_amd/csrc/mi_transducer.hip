@@ -65,7 +65,7 @@ namespace {
 // ----------------------------------------------------------------------------------------
 extern "C" {
 
-int mi_transducer_abi_version(void) { return 18; }
+int mi_transducer_abi_version(void) { return 17; }
 
 int mi_transducer_workspace_bytes(int B, int T, int U, int D, size_t* out_bytes) {
   Layout L;
@@ -181,8 +181,6 @@ int mi_tdt_forward(const void* acts, int act_dtype, const int64_t* labels, const
   st = check_common(acts, act_dtype, labels, act_lens, label_lens, B, T, U, V, D, blank, workspace, workspace_bytes,
                     stream, &c);
   if (st) return st;
-  // the TDT lattice and cell kernels read a cell's arc log-probs as one record, the plain RNNT kernels plane by plane
-  c.arc_ap = use_plain_rnnt ? 0 : c.L.AP;
   if ((st = run_denom(c))) return st;
   // omega branch (gpu_rnnt.py:607-622): the plain RNNT recursion over the token logits
   if (use_plain_rnnt) return run_rnnt_lattice(c, costs, fastemit_lambda, with_betas, 0, prefill_grads);
@@ -243,7 +241,6 @@ int mi_tdt_split_forward(const void* label_acts, const void* duration_acts, int 
   st = check_common(label_acts, act_dtype, labels, act_lens, label_lens, B, T, U, V, 0, blank, workspace,
                     workspace_bytes, stream, &c, 0, D);
   if (st) return st;
-  c.arc_ap = use_plain_rnnt ? 0 : c.L.AP;
   if ((st = run_denom(c))) return st;
   if (use_plain_rnnt) return run_rnnt_lattice(c, costs, fastemit_lambda, with_betas, 0, prefill_label_grads);
   if ((st = run_tdt_duration_planes(c, duration_acts, D))) return st;
@@ -436,13 +433,12 @@ int mi_transducer_length_maxima(const int64_t* act_lens, const int64_t* label_le
 }
 
 int mi_transducer_denominators(const void* acts, int act_dtype, const int64_t* labels, const int64_t* act_lens,
-                               const int64_t* label_lens, int B, int T, int U, int V, int D, int use_plain_rnnt,
-                               int blank, void* workspace, size_t workspace_bytes, void* stream) {
+                               const int64_t* label_lens, int B, int T, int U, int V, int D, int blank,
+                               void* workspace, size_t workspace_bytes, void* stream) {
   Common c;
   int st = check_common(acts, act_dtype, labels, act_lens, label_lens, B, T, U, V, D, blank, workspace,
                         workspace_bytes, stream, &c);
   if (st) return st;
-  c.arc_ap = (D > 0 && !use_plain_rnnt) ? c.L.AP : 0;
   return run_denom(c);
 }
 

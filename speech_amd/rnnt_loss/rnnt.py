@@ -107,16 +107,14 @@ def zero_padding(grads, act_lens, label_lens):
     _native.check_status(status, "zero_padding")
 
 
-def denominators(acts, labels, act_lens, label_lens, blank, workspace, num_durations=0, plain_rnnt=False):
-    """First stage of a forward call: log-softmax denominators and gathered arc log-probs into workspace.  With
-    durations, plain_rnnt says which lattice follows: tdt_lattice (False) or rnnt_lattice (True, the omega branch)."""
+def denominators(acts, labels, act_lens, label_lens, blank, workspace, num_durations=0):
+    """First stage of a forward call: log-softmax denominators and gathered arc log-probs into workspace."""
     _require_gpu(acts, "denominators")
     B, T, U, VD = acts.shape
     with torch.cuda.device(acts.device):
         status = _native.lib().mi_transducer_denominators(
             _ptr(acts), _dtype_code(acts), _labels_ptr(labels), _ptr(act_lens), _ptr(label_lens), B, T, U,
-            VD - num_durations, num_durations, int(bool(plain_rnnt)), int(blank), _ptr(workspace), workspace.numel(),
-            _stream(acts.device),
+            VD - num_durations, num_durations, int(blank), _ptr(workspace), workspace.numel(), _stream(acts.device),
         )  # fmt: skip
     _native.check_status(status, "Could not calculate forward scores")
 

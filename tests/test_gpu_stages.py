@@ -49,14 +49,6 @@ def test_denominators_then_lattice_is_the_forward_call(with_betas):
     assert torch.equal(whole, split)
     c_ref, _, _ = oracle.tdt_loss(rnnt_x, labels, al, ll, V - 1, durations, 0.05)
     np.testing.assert_allclose(split.cpu().numpy(), c_ref, rtol=1e-6)
-    # the omega branch of TDT: the plain RNNT lattice over the token logits of the same rows; the denominators are
-    # told, because the two lattices read the arc log-probs in different arrangements
-    rnnt.tdt_forward(acts, lab, ald, lld, whole, V - 1, durations, 0.0, 0.05, True, with_betas, ws1)
-    rnnt.denominators(acts, lab, ald, lld, V - 1, ws2, 3, plain_rnnt=True)
-    rnnt.rnnt_lattice(ald, lld, split, B, T, U, 0.0, with_betas, ws2, 3)
-    assert torch.equal(whole, split)
-    c_ref, _, _ = oracle.rnnt_loss(np.ascontiguousarray(rnnt_x[..., :V]), labels, al, ll, V - 1, 0.0, 0.0)
-    np.testing.assert_allclose(split.cpu().numpy(), c_ref, rtol=1e-6)
 
 
 def test_combined_tdt_function_level_seam():
