@@ -279,3 +279,27 @@ def test_function_level_seams_take_riders_by_themselves(omega):
         out[threshold] = res
     for a, b in zip(out[0], out[1 << 40]):
         assert torch.isfinite(a).all() and torch.equal(a, b)
+
+
+def test_random_shapes_with_and_without_riders():
+    """Seeded random shapes, lengths, dtypes and vocabulary sizes of every row-length class through the function-level
+    seam: with riders the costs and gradients are bit-identical to the plain calls, and the forward call touched
+    padding only."""
+    rng = np.random.RandomState(20240607)
+    Vs = [5, 17, 65, 129, 257, 513, 1025, 2049, 4097, 8193, 16385]
+    for it in range(45):
+        kind = ["rnnt", "tdt", "multiblank"][it % 3]
+        B, T, U = int(rng.randint(1, 6)), int(rng.randint(1, 200)), int(rng.randint(2, 60))
+        V = Vs[(it // 3) % len(Vs)] + {"rnnt": 0, "tdt": len(DURATIONS), "multiblank": len(BIG_BLANKS)}[kind]
+        if B * T * U * V > 2.0e7:
+            T = max(1, int(2.0e7 / (B * U * V)))
+        dtype = [torch.float32, torch.bfloat16, torch.float16][(it // 3) % 3]
+        acts, labels, al, ll = make(1000 + it, B, T, U, V, dtype)
+        case = "%s B=%d T=%d U=%d V=%d %s" % (kind, B, T, U, V, dtype)
+        plain = run(kind, acts, labels, al, ll, prefill=False)
+        ws = rnnt.new_workspace(acts, {"rnnt": 0, "tdt": len(DURATIONS), "multiblank": len(BIG_BLANKS)}[kind])
+        ridden = run(kind, acts, labels, al, ll, prefill=True, ws=ws)
+        assert torch.equal(plain[0], ridden[0]), case
+        assert torch.equal(plain[1], ridden[1]), case
+        assert torch.isfinite(ridden[1].float()).all(), case
+        check_forward_touched_padding_only(ridden[2], al, ll)
