@@ -33,9 +33,9 @@ constexpr int kScaleMaxBlocks = 2048;  // exponent tracks the scaled lattice ker
 // An item is 2^prefill_log_rows rows of one frame (b, t), items are numbered in memory order, and item i is the
 // (i / kFillMaxRiders)-th item of virtual rider i % kFillMaxRiders: it is done iff  i / kFillMaxRiders <
 // progress[i % kFillMaxRiders].  A launch has a power of two of real riders, each standing for the virtual riders
-// congruent to it.  The first two blocks are cleared by pass 1 and stamped with an epoch that changes with every
-// call, so what an earlier call left there is not mistaken for this call's -- also not in a captured graph, where
-// the epoch is frozen.
+// congruent to it.  Pass 1 clears the whole segment, and the first two blocks are stamped with an epoch that changes
+// with every call, so what an earlier call left there is not mistaken for this call's -- also not in a captured
+// graph, where the epoch is frozen -- and a record that no rider of this call wrote says that nothing is filled.
 constexpr int kFillMaxLattice = 256;
 constexpr int kFillMaxRiders = 4096;
 constexpr int kFillProgress = 2 * kFillMaxLattice;

@@ -39,7 +39,7 @@ def make(seed, B, T, U, V, dtype, full=False):
     return acts, labels, torch.tensor(al, device=DEV), torch.tensor(ll, device=DEV)
 
 
-def run(kind, acts, labels, al, ll, prefill, ws=None, scale=None):
+def run(kind, acts, labels, al, ll, prefill, ws=None, scale=None, mode=None):
     """(costs, grads, buffer as the forward call left it) through the function-level seam."""
     B, T, U, V = acts.shape
     D = {"rnnt": 0, "tdt": len(DURATIONS), "multiblank": len(BIG_BLANKS)}[kind]
@@ -47,7 +47,7 @@ def run(kind, acts, labels, al, ll, prefill, ws=None, scale=None):
     costs = torch.empty(B, dtype=torch.float32, device=DEV)
     grads = torch.full_like(acts, float("nan"))
     pre = grads if prefill else None
-    mode = 2 if prefill else 0
+    mode = (2 if prefill else 0) if mode is None else mode
     if kind == "rnnt":
         rnnt.rnnt_forward(acts, labels, al, ll, costs, V - 1, 0.01, True, ws, pre)
         after_forward = grads.clone()
@@ -303,3 +303,18 @@ def test_random_shapes_with_and_without_riders():
         assert torch.equal(plain[1], ridden[1]), case
         assert torch.isfinite(ridden[1].float()).all(), case
         check_forward_touched_padding_only(ridden[2], al, ll)
+
+
+@pytest.mark.parametrize("kind", ["rnnt", "tdt", "multiblank"])
+def test_a_record_of_an_earlier_call_is_not_believed(kind):
+    """A workspace whose last call had riders serves a forward call without a gradient buffer; a backward call that is
+    nevertheless told to consult the record must find it empty and write every padded cell itself."""
+    V = 1025 + {"rnnt": 0, "tdt": len(DURATIONS), "multiblank": len(BIG_BLANKS)}[kind]
+    acts, labels, al, ll = make(77, 4, 120, 40, V, torch.float32)
+    ws = rnnt.new_workspace(acts, {"rnnt": 0, "tdt": len(DURATIONS), "multiblank": len(BIG_BLANKS)}[kind])
+    first = run(kind, acts, labels, al, ll, prefill=True, ws=ws)
+    assert (~torch.isnan(first[2])).any(), "the riders of the first call were expected to fill something"
+    plain = run(kind, acts, labels, al, ll, prefill=False)
+    again = run(kind, acts, labels, al, ll, prefill=False, ws=ws, mode=2)
+    assert torch.isnan(again[2]).all()  # no riders: the forward call left the buffer alone
+    assert torch.equal(plain[0], again[0]) and torch.equal(plain[1], again[1])
