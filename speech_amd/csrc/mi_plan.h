@@ -122,8 +122,13 @@ inline GridDiv make_griddiv(int nchunks, int T) {
 }
 
 
+// Consecutive workgroups that one XCD takes per turn (logical_block, mi_device.inc).  Measured on the fwd+bwd step
+// with riders (us; B=16, T=375, U=121, V=1025 fp32 / the same as TDT / as multi-blank / B=32, T=750, U=201 bf16 /
+// V=16385): 512 -> 1110 / 1181 / 1110 / 3845 / 4996; 1024 -> 1116 / 1186 / 1125 / 3880 / 4990; at the first shape
+// 32, 128, 256, 384, 640, 768, 2048, 4096 -> 1123, 1120, 1117, 1115, 1117, 1115, 1133, 1152 (long turns leave XCDs
+// idle where an utterance's padding begins; short ones lose the linear walk).
 #ifndef MI_XCD_SPAN
-#define MI_XCD_SPAN 1024
+#define MI_XCD_SPAN 512
 #endif
 
 struct TdtParams {
