@@ -130,6 +130,15 @@ inline GridDiv make_griddiv(int nchunks, int T) {
 #ifndef MI_XCD_SPAN
 #define MI_XCD_SPAN 512
 #endif
+// The gradient pass over 16-bit rows wants shorter turns (its workgroups hold four rows of 2 KB where the fp32 ones
+// hold two of 4 KB): B=32, T=750, U=201, V=1025 bf16: 32 / 64 / 128 / 256 / 512 -> 2556 / 2536 / 2547 / 2575 / 2601 us
+// (step 3.76 against 3.83 ms); B=16, T=375, U=121 bf16: 361 / 360 / 359 / 363 / 378 us; the fp32 shapes all lose below
+// 512 (T=750, U=201 fp32: 5413 / 5476 / 5328 us at 128 / 256 / 512).  Pass 1 does not care (1038 ... 1043 us).
+// MI_XCD_SPAN is a multiple of it (grids are padded to a multiple of 8 * MI_XCD_SPAN).
+#ifndef MI_XCD_SPAN_16
+#define MI_XCD_SPAN_16 128
+#endif
+static_assert(MI_XCD_SPAN % MI_XCD_SPAN_16 == 0, "one grid padding must serve both turn lengths");
 
 struct TdtParams {
   int D;
