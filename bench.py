@@ -41,9 +41,9 @@ HBM_PEAK_GBPS = 8000.0  # MI355X HBM3E, published peak
 # this script, scaled by what the same counters read for mi_transducer_copy_probe of known size
 # (summaries under profiles/).  None = not measured for that workload.
 MEASURED_TRAFFIC_BYTES = {
-    # profiles/transducer_kernels_cfg2_hbm_traffic.md: fetch 1.6485 GB + write 2.6653 GB (the lattice launch, whose
+    # profiles/transducer_kernels_cfg2_hbm_traffic.md: fetch 1.6595 GB + write 2.6651 GB (the lattice launch, whose
     # riders zero-fill part of the padding, writes another 0.33 GB)
-    "cfg2_rnnt_B16_T375_U121_V1025_f32": int((804938 * 2.0 + 2602843) * 1024),
+    "cfg2_rnnt_B16_T375_U121_V1025_f32": int((810335 * 2.0 + 2602601) * 1024),
 }
 
 
