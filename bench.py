@@ -4,11 +4,16 @@
 A step is one forward + backward of the loss module over one resident batch:
     costs = loss(acts, labels, act_lens, label_lens); costs.sum().backward()
 on the north-star workload (RNNT, B=16, T=375, U+1=121, V=1025, fp32, variable
-lengths), inputs already in HBM.  Prints ONE JSON line:
+lengths), inputs already in HBM.  The timed steps are training steps, not replays: every step gets length tensors it
+has not seen (so the module's shape-vs-lengths check runs, with its read-back and host wait, as it does for a fresh
+batch) and the logits alternate between two buffers (so no step starts on what the step before left in the
+last-level cache).  The same loop over one set of tensors is timed beside it (`whole_job.same_tensors_ms_per_step`).
+Prints ONE JSON line:
   value        logit elements per second (B*T*U*V / step time)
   roofline     the gradient pass (the dominant kernel; its name for this shape is reported):
                algorithmic bytes per launch / its mean duration, measured with HIP events around
-               the launches of the timed steps
+               its launches in a second pass over the same steps (an event pair costs queue time, so
+               the steps that give ms_per_step carry none)
   cpu_baseline the C restatement of the reference's CPU path on a bounded sample, host cores (all threads, one
                thread, and the interpreted per-cell restatement at configuration 1)
   other_workloads  configurations 3, 4, 5 and the multi-blank one: median ms/step, bytes, fraction of peak
@@ -40,11 +45,16 @@ HBM_PEAK_GBPS = 8000.0  # MI355X HBM3E, published peak
 # HBM bytes per launch of the gradient-pass kernel from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of
 # this script, scaled by what the same counters read for mi_transducer_copy_probe of known size
 # (summaries under profiles/).  None = not measured for that workload.
-MEASURED_TRAFFIC_BYTES = {
-    # profiles/transducer_kernels_cfg2_hbm_traffic.md: fetch 1.6595 GB + write 2.6651 GB (the lattice launch, whose
-    # riders zero-fill part of the padding, writes another 0.33 GB)
-    "cfg2_rnnt_B16_T375_U121_V1025_f32": int((810335 * 2.0 + 2602601) * 1024),
+MEASURED_TRAFFIC_KIB = {
+    # workload: (FETCH_SIZE, WRITE_SIZE) of the gradient-pass kernel in KiB per dispatch, and the factors the same
+    # counters need to read a 1 GiB copy right (profiles/transducer_kernels_<cfg>_hbm_traffic.md)
 }
+TRAFFIC_SCALE = (2.0, 1.0)
+
+
+def measured_traffic(name):
+    kib = MEASURED_TRAFFIC_KIB.get(name)
+    return None if kib is None else int((kib[0] * TRAFFIC_SCALE[0] + kib[1] * TRAFFIC_SCALE[1]) * 1024)
 
 
 def parse_args():
@@ -58,9 +68,9 @@ def parse_args():
     ap.add_argument("--no-graph", action="store_true", help="skip the HIP-graph replay timing of the same step")
     ap.add_argument("--no-other-workloads", action="store_true",
                     help="skip the short runs of the other benchmark configurations (default run of workload 1 only)")
-    ap.add_argument("--lattice", choices=["auto", "log", "scaled"], default="auto",
-                    help="lattice kernels: auto = the library's default per loss, log = always the log-domain "
-                         "recursions, scaled = the probability-domain recursions wherever the shape allows (A/B timing)")
+    ap.add_argument("--same-tensors", action="store_true",
+                    help="headline loop over ONE set of tensors (the length check is then remembered and pass 1 starts "
+                         "in the last step's cache tail); default: fresh length tensors and alternating logits buffers")
     ap.add_argument("--cpu-sample-utterances", type=int, default=16)
     return ap.parse_args()
 
@@ -160,6 +170,43 @@ def cpu_baseline_logprobs(cfg, acts, labels, act_lens, label_lens, g_target, g_b
         "sample": f"first {n_utt} of {cfg.B} utterances of the same batch, full T x U x V, forward + backward, "
                   f"{dt:.2f} s wall (numpy, float64)",
     }  # fmt: skip
+
+
+def median(sorted_values):
+    n = len(sorted_values)
+    return sorted_values[n // 2] if n % 2 else 0.5 * (sorted_values[n // 2 - 1] + sorted_values[n // 2])
+
+
+def run_steps(torch, step_fn, bufs, act_lens, label_lens, steps, fresh):
+    """`steps` forward + backward steps, each timed by the stream events on either side of it.
+    step_fn(acts, act_lens, label_lens) -> costs.  fresh (a training loop): every step is given length tensors of its
+    own (cloned here, before the clock starts, so the module has not seen them and checks them against the shape as
+    it must for a new batch) and the next of the logits buffers in `bufs`; otherwise one set of tensors serves
+    every step.  Returns (sorted per-step ms, wall seconds, event ms over the whole loop, last costs)."""
+    if fresh:
+        lens = [(act_lens.clone(), label_lens.clone()) for _ in range(steps)]
+    else:
+        lens = [(act_lens, label_lens)] * steps
+    marks = [torch.cuda.Event(enable_timing=True) for _ in range(steps + 1)]
+    costs = None
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    marks[0].record()
+    for i in range(steps):
+        costs = step_fn(bufs[i % len(bufs)] if fresh else bufs[0], *lens[i])
+        marks[i + 1].record()
+    torch.cuda.synchronize()
+    wall = time.perf_counter() - t0
+    per_step = sorted(marks[i].elapsed_time(marks[i + 1]) for i in range(steps))
+    return per_step, wall, marks[0].elapsed_time(marks[-1]), costs
+
+
+PROTOCOLS = {
+    True: "training steps: length tensors the module has not seen (its shape check runs every step) and two "
+          "alternating logits buffers",
+    False: "one set of tensors for every step (the length check is remembered after the first, and pass 1 starts on "
+           "what the last step left in the last-level cache)",
+}  # fmt: skip
 
 
 def riders_filled_bytes(torch, cfg, acts, labels, act_lens, label_lens, reps=5):
@@ -265,33 +312,26 @@ def other_workloads(torch, dev, indices, steps=8, warmup=3):
             loss = RNNTLossNumba(blank=cfg.blank, reduction='none', fastemit_lambda=cfg.fastemit_lambda,
                                  clamp=cfg.clamp)  # fmt: skip
         nbytes = synthetic.algorithmic_bytes(cfg, act_lens, label_lens)
+        bufs = [acts, acts.detach().clone().requires_grad_(True)]
 
-        def step():
-            acts.grad = None
-            costs = loss(acts, labels, act_lens, label_lens)
+        def step(a, al, ll):
+            a.grad = None
+            costs = loss(a, labels, al, ll)
             costs.sum().backward()
             return costs
 
-        for _ in range(warmup):
-            step()
-        marks = [torch.cuda.Event(enable_timing=True) for _ in range(steps + 1)]
-        torch.cuda.synchronize()
-        marks[0].record()
-        for i in range(steps):
-            costs = step()
-            marks[i + 1].record()
-        torch.cuda.synchronize()
+        run_steps(torch, step, bufs, act_lens, label_lens, warmup, True)
+        per_step, _, _, costs = run_steps(torch, step, bufs, act_lens, label_lens, steps, True)
         assert bool(torch.isfinite(costs.float()).all()), "non-finite costs"
-        per_step = sorted(marks[i].elapsed_time(marks[i + 1]) for i in range(steps))
-        ms = 0.5 * (per_step[(steps - 1) // 2] + per_step[steps // 2])
+        ms = median(per_step)
         # a second pass with every pipeline kernel bracketed by events (not part of ms_per_step: the brackets cost
         # queue time): where the step goes, and how close the dominant kernel, the gradient pass, is to the HBM peak
         _native.profile_enable(steps)
-        for _ in range(steps):
-            step()
-        torch.cuda.synchronize()
+        run_steps(torch, step, bufs, act_lens, label_lens, steps, True)
         kernels = {k: v[0] / max(v[1], 1) for k, v in _native.profile_read().items()}
         _native.profile_disable()
+        for a in bufs:
+            a.grad = None
         grad_ms = kernels.get("gradient_pass", 0.0)
         riders_bytes = riders_filled_bytes(torch, cfg, acts.detach(), labels, act_lens, label_lens)
         out.append({
@@ -303,8 +343,10 @@ def other_workloads(torch, dev, indices, steps=8, warmup=3):
             "riders_filled_bytes": riders_bytes,
             "gradient_pass_frac_of_peak": (((nbytes["grad_stream"] - riders_bytes) / (grad_ms * 1e-3) / 1e9 / HBM_PEAK_GBPS)
                                            if grad_ms else None),
+            "gradient_pass_traffic_bytes": measured_traffic(cfg.name),
+            "protocol": PROTOCOLS[True],
         })  # fmt: skip
-        del acts, costs, loss
+        del acts, bufs, costs, loss
         torch.cuda.empty_cache()
     return out
 
@@ -413,7 +455,6 @@ def main():
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
     _native.lib()  # fail now if the HIP library is missing
-    _native.check_status(_native.lib().mi_transducer_set_lattice_mode({"auto": 0, "log": 1, "scaled": 2}[args.lattice]), "lattice mode")
 
     cfg, acts, labels, act_lens, label_lens = synthetic.make_inputs(args.workload, device=dev, generate_on_device=True)
     if args.op == "joint":
@@ -430,9 +471,9 @@ def main():
         loss = RNNTLossNumba(blank=cfg.blank, reduction='none', fastemit_lambda=cfg.fastemit_lambda, clamp=cfg.clamp)
     nbytes = synthetic.algorithmic_bytes(cfg, act_lens, label_lens)
 
-    def step():
-        acts.grad = None
-        costs = loss(acts, labels, act_lens, label_lens)
+    def step(a, al, ll):
+        a.grad = None
+        costs = loss(a, labels, al, ll)
         costs.sum().backward()
         return costs
 
@@ -451,44 +492,34 @@ def main():
         nbytes = dict(nbytes)
         nbytes["total"] = 2 * nbytes["c_valid"] * cfg.V * s_in + nbytes["cells"] * cfg.V * s_in + 16 * nbytes["cells"]
 
-        def step():  # noqa: F811
-            acts.grad = None
-            target_scores, blank_scores = rnnt_logprobs(acts, labels, cfg.blank, act_lens, label_lens)
+        def step(a, al, ll):  # noqa: F811
+            a.grad = None
+            target_scores, blank_scores = rnnt_logprobs(a, labels, cfg.blank, al, ll)
             torch.autograd.backward([target_scores, blank_scores], [g_target, g_blank])
             return blank_scores
 
-    for _ in range(args.warmup):
-        step()
-    torch.cuda.synchronize()
-
-    # the timed region: only the dominant kernel is bracketed by events (an event pair costs
-    # a few microseconds of queue time; the other kernels are timed in a separate pass below)
-    _native.profile_enable(args.steps, ["gradient_pass"])
-    marks = [torch.cuda.Event(enable_timing=True) for _ in range(args.steps + 1)]
-    torch.cuda.synchronize()
-    t0 = time.perf_counter()
-    marks[0].record()
-    for i in range(args.steps):
-        costs = step()
-        marks[i + 1].record()
-    torch.cuda.synchronize()
-    wall = time.perf_counter() - t0
-    kernels = _native.profile_read()
-    per_step = sorted(marks[i].elapsed_time(marks[i + 1]) for i in range(args.steps))
-    median_ms = per_step[len(per_step) // 2] if len(per_step) % 2 else 0.5 * (per_step[len(per_step) // 2 - 1] + per_step[len(per_step) // 2])
-    # per-kernel breakdown, outside the timed region
-    _native.profile_enable(args.steps)
-    for _ in range(args.steps):
-        step()
-    torch.cuda.synchronize()
-    breakdown = _native.profile_read()
-    _native.profile_disable()
+    bufs = [acts, acts.detach().clone().requires_grad_(True)]
+    fresh = not args.same_tensors
+    run_steps(torch, step, bufs, act_lens, label_lens, args.warmup, fresh)
+    # the timed region: nothing but the steps (no kernel is bracketed by events here)
+    per_step, wall, event_ms, costs = run_steps(torch, step, bufs, act_lens, label_lens, args.steps, fresh)
+    assert bool(torch.isfinite(costs).all()), "non-finite costs"
     # the headline is the MEDIAN step (stream events between the steps of the one timed loop); the mean of the same
     # loop by the host clock and by the events is reported beside it
+    ms_per_step = median(per_step)
     mean_wall_ms = wall * 1e3 / args.steps
-    event_ms_per_step = marks[0].elapsed_time(marks[-1]) / args.steps
-    ms_per_step = median_ms
-    assert bool(torch.isfinite(costs).all()), "non-finite costs"
+    event_ms_per_step = event_ms / args.steps
+    # the same loop under the other protocol, for comparison
+    run_steps(torch, step, bufs, act_lens, label_lens, min(args.warmup, 2), not fresh)
+    other_protocol_ms = median(run_steps(torch, step, bufs, act_lens, label_lens, args.steps, not fresh)[0])
+    # per-kernel durations from a pass of their own: every pipeline kernel bracketed by a pair of HIP events on its
+    # stream (the brackets cost queue time, so the steps above carry none)
+    _native.profile_enable(args.steps)
+    run_steps(torch, step, bufs, act_lens, label_lens, args.steps, fresh)
+    kernels = breakdown = _native.profile_read()
+    _native.profile_disable()
+    bufs[1].grad = None
+    del bufs
 
     # copy yardstick: 1 GiB device-to-device
     n = 1 << 30
@@ -552,6 +583,8 @@ def main():
             "min_ms_per_step": per_step[0],
             "max_ms_per_step": per_step[-1],
             "timing": "ms_per_step = median over the timed steps of the stream-event interval of each step",
+            "protocol": PROTOCOLS[fresh],
+            ("same_tensors_ms_per_step" if fresh else "training_steps_ms_per_step"): other_protocol_ms,
         },
         "roofline": {
             "kernel": plan["gradient"],
@@ -560,12 +593,13 @@ def main():
             "peak": HBM_PEAK_GBPS,
             "unit": "GB/s",
             "frac": achieved / HBM_PEAK_GBPS,
-            "traffic": None if logprobs else MEASURED_TRAFFIC_BYTES.get(cfg.name),
+            "traffic": None if logprobs else measured_traffic(cfg.name),
             "algorithmic_bytes_per_launch": grad_bytes,
             "padding_zero_filled_by": "this kernel, less what the riders of the lattice launch did",
             "riders_filled_bytes": riders_bytes,
             "avg_launch_ms": grad_avg_s * 1e3,
             "launches": grad_n,
+            "timed_in": "a second pass over the same steps with every pipeline kernel bracketed by HIP events",
         },
         "kernels": {k: (ms / max(n_, 1)) for k, (ms, n_) in breakdown.items()},
         "plan": plan,

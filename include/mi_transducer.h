@@ -45,6 +45,15 @@ extern "C" {
 #define MI_DTYPE_BF16 1
 #define MI_DTYPE_F16 2
 
+/* `riders` of the combined forward + backward entry points (mi_*_loss): whether the lattice launch of the call
+ * carries the extra workgroups that zero-fill gradient padding while the recursion runs (see prefill_grads of
+ * mi_rnnt_forward).  AUTO: only for gradients of 32 MiB and more (below that a step is bound by its launches).  The
+ * results are the same bits either way; any other value is invalid.  A per-call argument: the library keeps no
+ * setting that changes what a call computes or launches. */
+#define MI_RIDERS_AUTO (-1)
+#define MI_RIDERS_OFF 0
+#define MI_RIDERS_ON 1
+
 #define MI_TRANSDUCER_MAX_U 1024
 #define MI_TRANSDUCER_MAX_DURATIONS 16
 #define MI_TRANSDUCER_MAX_BIG_BLANKS 8      /* multi-blank: big blanks beside the standard blank */
@@ -70,7 +79,9 @@ int mi_transducer_workspace_bytes(int B, int T, int U, int D, size_t* out_bytes)
  * compute units busy and leaves HBM idle; given the buffer, the lattice launch carries extra workgroups that
  * zero-fill the gradient of padded cells meanwhile (part of what zeros_like + `grads *= 0` do up front in the
  * reference, rnnt_pytorch.py:58, gpu_rnnt.py:156), stop when the lattice ends, and record in the workspace how far
- * they got.  The backward call is then given padding_zeroed = 2.  Ignored when with_betas == 0. */
+ * they got.  The backward call is then given padding_zeroed = 2.  Ignored when with_betas == 0, and for the shapes
+ * whose gradient kernel cannot consult that record (rows beyond 8192 16-byte vectors, more than 128 utterances).
+ * Whether a problem is large enough for this to pay is the caller's decision (see MI_RIDERS_AUTO). */
 int mi_rnnt_forward(const void* acts, int act_dtype, const int64_t* labels, const int64_t* act_lens,
                     const int64_t* label_lens, float* costs, int B, int T, int U, int V, int blank,
                     float fastemit_lambda, int with_betas, void* prefill_grads, void* workspace,
@@ -100,7 +111,7 @@ int mi_rnnt_backward(const void* acts, int act_dtype, const int64_t* labels, con
 int mi_rnnt_loss(const void* acts, int act_dtype, const int64_t* labels, const int64_t* act_lens,
                  const int64_t* label_lens, float* costs, void* grads, const float* grad_scale,
                  int grad_scale_stride, float grad_mul, int B, int T, int U, int V, int blank, float fastemit_lambda,
-                 float clamp, void* workspace, size_t workspace_bytes, void* stream);
+                 float clamp, int riders, void* workspace, size_t workspace_bytes, void* stream);
 
 /* mi_rnnt_loss without a workspace argument, for callers that cannot allocate one: code under HIP graph capture,
  * tight serving loops, harnesses that forbid hipMalloc.  It has no counterpart in the reference (whose wrapper
@@ -118,7 +129,7 @@ int mi_transducer_init(void);
 int mi_rnnt_loss_static(const void* acts, int act_dtype, const int64_t* labels, const int64_t* act_lens,
                         const int64_t* label_lens, float* costs, void* grads, const float* grad_scale,
                         int grad_scale_stride, float grad_mul, int B, int T, int U, int V, int blank,
-                        float fastemit_lambda, float clamp, void* stream);
+                        float fastemit_lambda, float clamp, int riders, void* stream);
 
 /* TDT.  acts is the COMBINED tensor [B,T,U,V+D]: V token logits (blank included)
  * followed by D duration logits, exactly what TDTLossNumba.forward receives
@@ -145,7 +156,7 @@ int mi_tdt_backward(const void* acts, int act_dtype, const int64_t* labels, cons
 int mi_tdt_loss(const void* acts, int act_dtype, const int64_t* labels, const int64_t* act_lens,
                 const int64_t* label_lens, float* costs, void* grads, const float* grad_scale, int grad_scale_stride,
                 float grad_mul, int B, int T, int U, int V, int D, const int32_t* durations_host, int blank,
-                float fastemit_lambda, float clamp, float sigma, int use_plain_rnnt, void* workspace,
+                float fastemit_lambda, float clamp, float sigma, int use_plain_rnnt, int riders, void* workspace,
                 size_t workspace_bytes, void* stream);
 
 /* TDT with the reference's function-level operands (tdt_loss_gpu, rnnt.py:239-255; GPUTDT.cost_and_grad /
@@ -173,8 +184,8 @@ int mi_tdt_split_loss(const void* label_acts, const void* duration_acts, int act
                       const int64_t* act_lens, const int64_t* label_lens, float* costs, void* label_grads,
                       void* duration_grads, const float* grad_scale, int grad_scale_stride, float grad_mul, int B,
                       int T, int U, int V, int D, const int32_t* durations_host, int blank, float fastemit_lambda,
-                      float clamp, float sigma, int use_plain_rnnt, void* workspace, size_t workspace_bytes,
-                      void* stream);
+                      float clamp, float sigma, int use_plain_rnnt, int riders, void* workspace,
+                      size_t workspace_bytes, void* stream);
 
 /* ---- multi-blank transducer ---------------------------------------------------------
  * Replaces rnnt.py:366-483 (multiblank_rnnt_loss_gpu) and what it drives:
@@ -201,7 +212,7 @@ int mi_multiblank_loss(const void* acts, int act_dtype, const int64_t* labels, c
                        const int64_t* label_lens, float* costs, void* grads, const float* grad_scale,
                        int grad_scale_stride, float grad_mul, int B, int T, int U, int V, int num_big_blanks,
                        const int32_t* big_blank_durations_host, int blank, float fastemit_lambda, float clamp,
-                       float sigma, void* workspace, size_t workspace_bytes, void* stream);
+                       float sigma, int riders, void* workspace, size_t workspace_bytes, void* stream);
 
 /* The two stages of a forward call on their own (mi_rnnt_forward = denominators + rnnt lattice,
  * mi_tdt_forward = denominators + tdt lattice), for callers that want to order other work between
@@ -363,8 +374,8 @@ int mi_transducer_length_maxima(const int64_t* act_lens, const int64_t* label_le
 
 /* ---- diagnostics ------------------------------------------------------------------------
  * Everything from here to the end of this header (mi_transducer_profile_*, mi_transducer_describe_plan,
- * mi_transducer_copy_probe, mi_transducer_set_lattice_mode, mi_transducer_scale_segment,
- * mi_transducer_prefill_record, mi_transducer_set_prefill_min_bytes) binds NO interface of the reference: these are aids for benchmarks, profiles and tests
+ * mi_transducer_copy_probe, mi_transducer_prefill_record) binds NO interface of the reference: these are aids for
+ * benchmarks, profiles and tests
  * of this library, and a drop-in user of the loss never calls them.
  *
  * Per-kernel timing of the launches a harness itself makes: after
@@ -378,7 +389,7 @@ int mi_transducer_length_maxima(const int64_t* act_lens, const int64_t* label_le
  * calls are safe from any thread, but launches from several threads are then counted into the same classes.  Leave
  * it disabled outside benchmarks (disabled, a launch only reads one flag). */
 #define MI_PROFILE_DENOM 0   /* denom_rows_kernel / denom_block_kernel / denom_gather_kernel */
-#define MI_PROFILE_LATTICE 1 /* rnnt_scaled_lattice_kernel / rnnt_lattice_kernel / tdt_lattice_pair_kernel / tdt_lattice_kernel */
+#define MI_PROFILE_LATTICE 1 /* rnnt_lattice_kernel / tdt_lattice_pair_kernel / tdt_lattice_kernel */
 #define MI_PROFILE_CELL 2    /* rnnt_cell_kernel / tdt_cell_kernel */
 #define MI_PROFILE_GRAD 3    /* grad_rows_kernel / grad_block_kernel / grad_stream_kernel */
 #define MI_PROFILE_ZERO 4    /* zero_padding_kernel */
@@ -401,19 +412,6 @@ int mi_transducer_describe_plan(int act_dtype, int B, int T, int U, int V, int D
  * counters and for the copy bandwidth the GPU reaches in practice. */
 int mi_transducer_copy_probe(const void* src, void* dst, size_t bytes, void* stream);
 
-/* Which lattice kernels the forward calls run (process-wide): 0 (the default) = per loss, whichever measured
- * faster; 1 = always the log-domain recursions; 2 = the scaled, probability-domain recursions wherever the shape
- * allows them (each returns to the log domain per utterance when its own checks ask for it).  For tests that hold
- * one against the other and for A/B timing. */
-int mi_transducer_set_lattice_mode(int mode);
-
-/* Where a workspace of this shape keeps, per utterance, the word that says which format the last RNNT lattice
- * kernel left alphas and betas in (0 = natural logs, 1 = scaled probabilities): int32 number
- * `*format_word` of the `*ints_per_utterance` ints that start at byte `*offset_bytes + 4 * b * *ints_per_utterance`.
- * Host arithmetic only.  For tests that must know which of the two recursions produced a result. */
-int mi_transducer_scale_segment(int B, int T, int U, int D, size_t* offset_bytes, int* ints_per_utterance,
-                                int* format_word);
-
 /* Where a workspace of this shape keeps the record of what the riders of the last forward call with prefill_grads
  * zero-filled: `*words` int32 starting at byte `*offset_bytes`.  Rows of row_bytes bytes go `*rows_per_item` to an
  * item (the last item of a frame may be shorter), items are numbered in memory order over (b, t, item of the frame),
@@ -421,11 +419,6 @@ int mi_transducer_scale_segment(int B, int T, int U, int D, size_t* offset_bytes
  * benchmarks that report how many bytes moved from the gradient pass into the lattice launch, and for tests. */
 int mi_transducer_prefill_record(int B, int T, int U, int D, size_t row_bytes, size_t* offset_bytes, int* words,
                                  int* rows_per_item);
-
-/* A forward call given prefill_grads launches riders only if the gradient tensor has at least this many bytes
- * (process-wide; 32 MiB unless set): below that a step is bound by its launches.  Tests set it to 0 so that small
- * shapes run the riders too. */
-int mi_transducer_set_prefill_min_bytes(size_t bytes);
 
 #ifdef __cplusplus
 }

@@ -21,10 +21,11 @@ CPU_SOURCES = [os.path.join(CSRC_DIR, "mi_cpu.cpp")]
 CPU_ABI_VERSION = 1
 CXX_FLAGS = ["-O3", "-std=c++17", "-fPIC", "-shared", "-fopenmp", "-Wall", "-Wextra"]
 
-ABI_VERSION = 17
+ABI_VERSION = 18
 SUCCESS, INVALID_VALUE, LAUNCH_FAILURE, TOO_LARGE = 0, 1, 2, 3
 STATIC_WORKSPACE_BYTES = 64 << 20
 DTYPE_F32, DTYPE_BF16, DTYPE_F16 = 0, 1, 2
+RIDERS_AUTO, RIDERS_OFF, RIDERS_ON = -1, 0, 1  # `riders` of the combined mi_*_loss entry points
 
 HIPCC_FLAGS = [
     "--offload-arch=gfx950",
@@ -79,29 +80,29 @@ _SIGNATURES = {
     "mi_rnnt_backward": [_vp, _c_int, _vp, _vp, _vp, _vp, _vp, _c_int, _c_float, _c_int, _c_int, _c_int, _c_int,
                          _c_int, _c_int, _c_float, _c_float, _vp, _c_size_t, _vp],
     "mi_rnnt_loss": [_vp, _c_int, _vp, _vp, _vp, _vp, _vp, _vp, _c_int, _c_float, _c_int, _c_int, _c_int, _c_int,
-                     _c_int, _c_float, _c_float, _vp, _c_size_t, _vp],
+                     _c_int, _c_float, _c_float, _c_int, _vp, _c_size_t, _vp],
     "mi_transducer_init": [],
     "mi_rnnt_loss_static": [_vp, _c_int, _vp, _vp, _vp, _vp, _vp, _vp, _c_int, _c_float, _c_int, _c_int, _c_int, _c_int,
-                            _c_int, _c_float, _c_float, _vp],
+                            _c_int, _c_float, _c_float, _c_int, _vp],
     "mi_tdt_forward": [_vp, _c_int, _vp, _vp, _vp, _vp, _c_int, _c_int, _c_int, _c_int, _c_int, _vp, _c_int, _c_float,
                        _c_float, _c_int, _c_int, _vp, _vp, _c_size_t, _vp],
     "mi_tdt_backward": [_vp, _c_int, _vp, _vp, _vp, _vp, _vp, _c_int, _c_float, _c_int, _c_int, _c_int, _c_int,
                         _c_int, _c_int, _vp, _c_int, _c_float, _c_float, _c_float, _c_int, _vp, _c_size_t, _vp],
     "mi_tdt_loss": [_vp, _c_int, _vp, _vp, _vp, _vp, _vp, _vp, _c_int, _c_float, _c_int, _c_int, _c_int, _c_int,
-                    _c_int, _vp, _c_int, _c_float, _c_float, _c_float, _c_int, _vp, _c_size_t, _vp],
+                    _c_int, _vp, _c_int, _c_float, _c_float, _c_float, _c_int, _c_int, _vp, _c_size_t, _vp],
     "mi_tdt_split_forward": [_vp, _vp, _c_int, _vp, _vp, _vp, _vp, _c_int, _c_int, _c_int, _c_int, _c_int, _vp, _c_int,
                              _c_float, _c_float, _c_int, _c_int, _vp, _vp, _c_size_t, _vp],
     "mi_tdt_split_backward": [_vp, _c_int, _vp, _vp, _vp, _vp, _vp, _vp, _c_int, _c_float, _c_int, _c_int, _c_int,
                               _c_int, _c_int, _c_int, _vp, _c_int, _c_float, _c_float, _c_float, _c_int, _vp,
                               _c_size_t, _vp],
     "mi_tdt_split_loss": [_vp, _vp, _c_int, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _c_int, _c_float, _c_int, _c_int, _c_int,
-                          _c_int, _c_int, _vp, _c_int, _c_float, _c_float, _c_float, _c_int, _vp, _c_size_t, _vp],
+                          _c_int, _c_int, _vp, _c_int, _c_float, _c_float, _c_float, _c_int, _c_int, _vp, _c_size_t, _vp],
     "mi_multiblank_forward": [_vp, _c_int, _vp, _vp, _vp, _vp, _c_int, _c_int, _c_int, _c_int, _c_int, _vp, _c_int,
                               _c_float, _c_float, _c_int, _vp, _vp, _c_size_t, _vp],
     "mi_multiblank_backward": [_vp, _c_int, _vp, _vp, _vp, _vp, _vp, _c_int, _c_float, _c_int, _c_int, _c_int, _c_int,
                                _c_int, _c_int, _vp, _c_int, _c_float, _c_float, _c_float, _vp, _c_size_t, _vp],
     "mi_multiblank_loss": [_vp, _c_int, _vp, _vp, _vp, _vp, _vp, _vp, _c_int, _c_float, _c_int, _c_int, _c_int, _c_int,
-                           _c_int, _vp, _c_int, _c_float, _c_float, _c_float, _vp, _c_size_t, _vp],
+                           _c_int, _vp, _c_int, _c_float, _c_float, _c_float, _c_int, _vp, _c_size_t, _vp],
     "mi_rnnt_logprobs_forward": [_vp, _c_int, _vp, _vp, _vp, _vp, _vp, _c_int, _c_int, _c_int, _c_int, _c_int, _vp,
                                  _c_size_t, _vp],
     "mi_rnnt_logprobs_backward": [_vp, _c_int, _vp, _vp, _vp, _vp, _vp, _vp, _c_int, _c_int, _c_int, _c_int, _c_int,
@@ -146,10 +147,7 @@ _SIGNATURES = {
     "mi_transducer_describe_plan": [_c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int,
                                     ctypes.c_char_p, _c_size_t],
     "mi_transducer_copy_probe": [_vp, _vp, _c_size_t, _vp],
-    "mi_transducer_set_lattice_mode": [_c_int],
-    "mi_transducer_scale_segment": [_c_int, _c_int, _c_int, _c_int, _vp, _vp, _vp],
     "mi_transducer_prefill_record": [_c_int, _c_int, _c_int, _c_int, _c_size_t, _vp, _vp, _vp],
-    "mi_transducer_set_prefill_min_bytes": [_c_size_t],
 }  # fmt: skip
 
 EXPORTED_SYMBOLS = tuple(_SIGNATURES)

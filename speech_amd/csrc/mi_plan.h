@@ -11,20 +11,6 @@
 #include "mi_transducer.h"
 
 constexpr int kCoefBase = 8;  // floats per cell in the coefficient buffer before the duration-gradient block
-// The scale segment of the workspace, per utterance, in ints (a multiple of four of them, so every header starts
-// on a 16-byte boundary):
-//   [0,1] 64-bit mark a pass-1 kernel leaves when an arc probability of the utterance is not a normal double
-//   [2,3] why the scaled lattice kernel took the log route (0: it did not), and its exponent spread
-//   [4]   format of the stored alphas / betas: 0 = natural logs, 1 = scaled probabilities
-//   [5]   binary exponent of the total probability Z = zm * 2^[5]          (format 1)
-//   [6,7] the double 1 / zm                                                 (format 1)
-//   then per block g of kScaleBlock anti-diagonals the pair {alpha exponent, beta exponent}: a stored value v of
-//   block g stands for v * 2^exponent
-constexpr int kScaleHeader = 8;
-constexpr int kScaleFormat = 4;  // index of the format word in the header
-constexpr int kScaleBlock = 8;
-constexpr int kScaleMaxBlocks = 2048;  // exponent tracks the scaled lattice kernel can hold in LDS
-
 // The prefill segment of the workspace, in ints.  While a lattice kernel runs, HBM idles; "riders" (extra workgroups
 // of the same launch) zero-fill the padded cells of the gradient meanwhile, as far as they get.
 //   [0, kFillMaxLattice)                  per lattice workgroup: (epoch << 13) | (id of the compute unit it runs on + 1)
@@ -58,9 +44,7 @@ struct Layout {
   int ND;   // number of anti-diagonals of the padded lattice = T+U-1
   int A;    // arc planes per diagonal row: blank, label, D duration log-probs
   int CS;   // floats per cell in the coefficient buffer
-  int SG;   // ints per utterance in the scale segment: kScaleHeader, then {alpha, beta} exponent per 8 diagonals
-  size_t off_denom, off_arcs, off_alphas, off_betas, off_ll, off_coef, off_scale, off_fill, total;
-  size_t off_arcp, total_scaled;  // total_scaled = total + the arc-probability segment of the scaled RNNT lattice
+  size_t off_denom, off_arcs, off_alphas, off_betas, off_ll, off_coef, off_fill, total;
 };
 
 inline size_t align256(size_t x) { return (x + 255) & ~(size_t)255; }
@@ -83,16 +67,8 @@ inline bool make_layout(int B, int T, int U, int D, Layout* L) {
   L->off_betas = off;  off = align256(off + skew * sizeof(double));
   L->off_ll = off;     off = align256(off + (size_t)B * 2 * sizeof(double));
   L->off_coef = off;   off = align256(off + cells * L->CS * sizeof(float));
-  // per utterance a header (which format the lattice is in, the total probability) followed by the binary exponents
-  // of the alpha and beta values of every block of kScaleBlock anti-diagonals of a scaled lattice
-  L->SG = kScaleHeader + 2 * ((L->ND / kScaleBlock + 3) & ~1);
-  L->off_scale = off;  off = align256(off + (size_t)B * L->SG * sizeof(int));
   L->off_fill = off;   off = align256(off + (size_t)kFillInts * sizeof(int));
   L->total = off;
-  // the scaled (probability-domain) RNNT lattice also wants the blank / label arc PROBABILITIES as doubles, skewed
-  // like `arcs`: a segment behind everything else that only a caller who asked for that lattice has to bring
-  L->off_arcp = off;   off = align256(off + (D == 0 ? skew * 2 * sizeof(double) : 0));
-  L->total_scaled = off;
   return true;
 }
 

@@ -65,13 +65,12 @@ namespace {
 // ----------------------------------------------------------------------------------------
 extern "C" {
 
-int mi_transducer_abi_version(void) { return 17; }
+int mi_transducer_abi_version(void) { return 18; }
 
 int mi_transducer_workspace_bytes(int B, int T, int U, int D, size_t* out_bytes) {
   Layout L;
   if (!out_bytes || !make_layout(B, T, U, D, &L)) return MI_TRANSDUCER_INVALID_VALUE;
-  // (the scaled RNNT lattice, lattice mode 2, keeps one more segment)
-  *out_bytes = g_lattice_mode.load(std::memory_order_relaxed) == 2 ? L.total_scaled : L.total;
+  *out_bytes = L.total;
   return MI_TRANSDUCER_SUCCESS;
 }
 
@@ -84,9 +83,8 @@ int mi_rnnt_forward(const void* acts, int act_dtype, const int64_t* labels, cons
   int st = check_common(acts, act_dtype, labels, act_lens, label_lens, B, T, U, V, 0, blank, workspace,
                         workspace_bytes, stream, &c);
   if (st) return st;
-  const unsigned long long mark = scaled_lattice_mark(c, with_betas);
-  if ((st = run_denom(c, mark))) return st;
-  return run_rnnt_lattice(c, costs, fastemit_lambda, with_betas, mark, with_betas ? prefill_grads : nullptr);
+  if ((st = run_denom(c))) return st;
+  return run_rnnt_lattice(c, costs, fastemit_lambda, with_betas, with_betas ? prefill_grads : nullptr);
 }
 
 int mi_rnnt_backward(const void* acts, int act_dtype, const int64_t* labels, const int64_t* act_lens,
@@ -108,13 +106,16 @@ int mi_rnnt_backward(const void* acts, int act_dtype, const int64_t* labels, con
 int mi_rnnt_loss(const void* acts, int act_dtype, const int64_t* labels, const int64_t* act_lens,
                  const int64_t* label_lens, float* costs, void* grads, const float* grad_scale,
                  int grad_scale_stride, float grad_mul, int B, int T, int U, int V, int blank, float fastemit_lambda,
-                 float clamp, void* workspace, size_t workspace_bytes, void* stream) {
-  // (the lattice launch zero-fills padded cells of grads while it runs; the gradient pass skips those)
+                 float clamp, int riders, void* workspace, size_t workspace_bytes, void* stream) {
+  if (!riders_arg_ok(riders)) return MI_TRANSDUCER_INVALID_VALUE;
+  // (with riders the lattice launch zero-fills padded cells of grads while it runs; the gradient pass skips those)
+  void* prefill = grads && riders_wanted(riders, B, T, U, V, act_dtype) ? grads : nullptr;
   int st = mi_rnnt_forward(acts, act_dtype, labels, act_lens, label_lens, costs, B, T, U, V, blank, fastemit_lambda,
-                           grads != nullptr, grads, workspace, workspace_bytes, stream);
+                           grads != nullptr, prefill, workspace, workspace_bytes, stream);
   if (st || !grads) return st;
   return mi_rnnt_backward(acts, act_dtype, labels, act_lens, label_lens, grads, grad_scale, grad_scale_stride,
-                          grad_mul, 2, B, T, U, V, blank, fastemit_lambda, clamp, workspace, workspace_bytes, stream);
+                          grad_mul, prefill ? 2 : 0, B, T, U, V, blank, fastemit_lambda, clamp, workspace,
+                          workspace_bytes, stream);
 }
 
 // ----------------------------------------------------------------------------------------
@@ -155,7 +156,7 @@ int mi_transducer_init(void) {
 int mi_rnnt_loss_static(const void* acts, int act_dtype, const int64_t* labels, const int64_t* act_lens,
                         const int64_t* label_lens, float* costs, void* grads, const float* grad_scale,
                         int grad_scale_stride, float grad_mul, int B, int T, int U, int V, int blank,
-                        float fastemit_lambda, float clamp, void* stream) {
+                        float fastemit_lambda, float clamp, int riders, void* stream) {
   Layout L;
   if (!make_layout(B, T, U, 0, &L)) return MI_TRANSDUCER_INVALID_VALUE;
   if (L.total > (size_t)MI_TRANSDUCER_STATIC_WORKSPACE_BYTES) return MI_TRANSDUCER_TOO_LARGE;
@@ -165,7 +166,7 @@ int mi_rnnt_loss_static(const void* acts, int act_dtype, const int64_t* labels, 
   // nothing in the workspace has to start at zero: every kernel writes what later kernels of the call read, and
   // what is left there by an earlier call is never read
   return mi_rnnt_loss(acts, act_dtype, labels, act_lens, label_lens, costs, grads, grad_scale, grad_scale_stride,
-                      grad_mul, B, T, U, V, blank, fastemit_lambda, clamp, ws, L.total, stream);
+                      grad_mul, B, T, U, V, blank, fastemit_lambda, clamp, riders, ws, L.total, stream);
 }
 
 int mi_tdt_forward(const void* acts, int act_dtype, const int64_t* labels, const int64_t* act_lens,
@@ -183,7 +184,7 @@ int mi_tdt_forward(const void* acts, int act_dtype, const int64_t* labels, const
   if (st) return st;
   if ((st = run_denom(c))) return st;
   // omega branch (gpu_rnnt.py:607-622): the plain RNNT recursion over the token logits
-  if (use_plain_rnnt) return run_rnnt_lattice(c, costs, fastemit_lambda, with_betas, 0, prefill_grads);
+  if (use_plain_rnnt) return run_rnnt_lattice(c, costs, fastemit_lambda, with_betas, prefill_grads);
   return run_tdt_lattice(c, costs, fastemit_lambda, with_betas, prm, prefill_grads);
 }
 
@@ -215,9 +216,10 @@ int mi_tdt_backward(const void* acts, int act_dtype, const int64_t* labels, cons
 int mi_tdt_loss(const void* acts, int act_dtype, const int64_t* labels, const int64_t* act_lens,
                 const int64_t* label_lens, float* costs, void* grads, const float* grad_scale, int grad_scale_stride,
                 float grad_mul, int B, int T, int U, int V, int D, const int32_t* durations_host, int blank,
-                float fastemit_lambda, float clamp, float sigma, int use_plain_rnnt, void* workspace,
+                float fastemit_lambda, float clamp, float sigma, int use_plain_rnnt, int riders, void* workspace,
                 size_t workspace_bytes, void* stream) {
-  void* prefill = grads;
+  if (!riders_arg_ok(riders)) return MI_TRANSDUCER_INVALID_VALUE;
+  void* prefill = grads && riders_wanted(riders, B, T, U, V + D, act_dtype) ? grads : nullptr;
   int st = mi_tdt_forward(acts, act_dtype, labels, act_lens, label_lens, costs, B, T, U, V, D, durations_host, blank,
                           fastemit_lambda, sigma, use_plain_rnnt, grads != nullptr, prefill, workspace, workspace_bytes,
                           stream);
@@ -242,7 +244,7 @@ int mi_tdt_split_forward(const void* label_acts, const void* duration_acts, int 
                     workspace_bytes, stream, &c, 0, D);
   if (st) return st;
   if ((st = run_denom(c))) return st;
-  if (use_plain_rnnt) return run_rnnt_lattice(c, costs, fastemit_lambda, with_betas, 0, prefill_label_grads);
+  if (use_plain_rnnt) return run_rnnt_lattice(c, costs, fastemit_lambda, with_betas, prefill_label_grads);
   if ((st = run_tdt_duration_planes(c, duration_acts, D))) return st;
   return run_tdt_lattice(c, costs, fastemit_lambda, with_betas, prm, prefill_label_grads);
 }
@@ -280,10 +282,11 @@ int mi_tdt_split_loss(const void* label_acts, const void* duration_acts, int act
                       const int64_t* act_lens, const int64_t* label_lens, float* costs, void* label_grads,
                       void* duration_grads, const float* grad_scale, int grad_scale_stride, float grad_mul, int B,
                       int T, int U, int V, int D, const int32_t* durations_host, int blank, float fastemit_lambda,
-                      float clamp, float sigma, int use_plain_rnnt, void* workspace, size_t workspace_bytes,
-                      void* stream) {
-  if ((label_grads == nullptr) != (duration_grads == nullptr)) return MI_TRANSDUCER_INVALID_VALUE;
-  void* prefill = label_grads;
+                      float clamp, float sigma, int use_plain_rnnt, int riders, void* workspace,
+                      size_t workspace_bytes, void* stream) {
+  if ((label_grads == nullptr) != (duration_grads == nullptr) || !riders_arg_ok(riders))
+    return MI_TRANSDUCER_INVALID_VALUE;
+  void* prefill = label_grads && riders_wanted(riders, B, T, U, V, act_dtype) ? label_grads : nullptr;
   int st = mi_tdt_split_forward(label_acts, duration_acts, act_dtype, labels, act_lens, label_lens, costs, B, T, U, V, D,
                                 durations_host, blank, fastemit_lambda, sigma, use_plain_rnnt, label_grads != nullptr,
                                 prefill, workspace, workspace_bytes, stream);
@@ -338,13 +341,15 @@ int mi_multiblank_loss(const void* acts, int act_dtype, const int64_t* labels, c
                        const int64_t* label_lens, float* costs, void* grads, const float* grad_scale,
                        int grad_scale_stride, float grad_mul, int B, int T, int U, int V, int num_big_blanks,
                        const int32_t* big_blank_durations_host, int blank, float fastemit_lambda, float clamp,
-                       float sigma, void* workspace, size_t workspace_bytes, void* stream) {
+                       float sigma, int riders, void* workspace, size_t workspace_bytes, void* stream) {
+  if (!riders_arg_ok(riders)) return MI_TRANSDUCER_INVALID_VALUE;
+  void* prefill = grads && riders_wanted(riders, B, T, U, V, act_dtype) ? grads : nullptr;
   int st = mi_multiblank_forward(acts, act_dtype, labels, act_lens, label_lens, costs, B, T, U, V, num_big_blanks,
-                                 big_blank_durations_host, blank, fastemit_lambda, sigma, grads != nullptr, grads,
+                                 big_blank_durations_host, blank, fastemit_lambda, sigma, grads != nullptr, prefill,
                                  workspace, workspace_bytes, stream);
   if (st || !grads) return st;
   return mi_multiblank_backward(acts, act_dtype, labels, act_lens, label_lens, grads, grad_scale, grad_scale_stride,
-                                grad_mul, 2, B, T, U, V, num_big_blanks, big_blank_durations_host, blank, fastemit_lambda,
+                                grad_mul, prefill ? 2 : 0, B, T, U, V, num_big_blanks, big_blank_durations_host, blank, fastemit_lambda,
                                 clamp, sigma, workspace, workspace_bytes, stream);
 }
 
@@ -387,20 +392,9 @@ int mi_transducer_export_lattice(const void* workspace, size_t workspace_bytes, 
   hipLaunchKernelGGL(export_lattice_kernel, dim3(grid), dim3(256), 0, (hipStream_t)stream,
                      (const float*)(ws + L.off_denom), (const double*)(ws + L.off_alphas),
                      (const double*)(ws + L.off_betas), (const double*)(ws + L.off_ll),
-                     D == 0 ? (const int*)(ws + L.off_scale) : nullptr, L.SG, act_lens, label_lens, denom, alphas, betas,
+                     act_lens, label_lens, denom, alphas, betas,
                      ll_forward, ll_backward, B, T, U, L.ND, L.Us, cells);
   return launch_status();
-}
-
-int mi_transducer_scale_segment(int B, int T, int U, int D, size_t* offset_bytes, int* ints_per_utterance,
-                                int* format_word) {
-  Layout L;
-  if (!offset_bytes || !ints_per_utterance || !format_word || !make_layout(B, T, U, D, &L))
-    return MI_TRANSDUCER_INVALID_VALUE;
-  *offset_bytes = L.off_scale;
-  *ints_per_utterance = L.SG;
-  *format_word = kScaleFormat;
-  return MI_TRANSDUCER_SUCCESS;
 }
 
 int mi_transducer_prefill_record(int B, int T, int U, int D, size_t row_bytes, size_t* offset_bytes, int* words,
@@ -411,17 +405,6 @@ int mi_transducer_prefill_record(int B, int T, int U, int D, size_t row_bytes, s
   *offset_bytes = L.off_fill + (size_t)kFillProgress * sizeof(int);
   *words = kFillMaxRiders;
   *rows_per_item = 1 << prefill_log_rows(row_bytes);
-  return MI_TRANSDUCER_SUCCESS;
-}
-
-int mi_transducer_set_prefill_min_bytes(size_t bytes) {
-  g_prefill_min_bytes.store(bytes, std::memory_order_relaxed);
-  return MI_TRANSDUCER_SUCCESS;
-}
-
-int mi_transducer_set_lattice_mode(int mode) {
-  if (mode < 0 || mode > 2) return MI_TRANSDUCER_INVALID_VALUE;
-  g_lattice_mode.store(mode, std::memory_order_relaxed);
   return MI_TRANSDUCER_SUCCESS;
 }
 
@@ -575,7 +558,7 @@ int mi_transducer_describe_plan(int act_dtype, int B, int T, int U, int V, int D
   else if (rows_R(c)) snprintf(grad, sizeof grad, "grad_rows_kernel<%s, R=%d, %s>", dt, rows_R(c), fused ? "fused" : "coef");
   else snprintf(grad, sizeof grad, "grad_stream_kernel<%s>", dt);
   const int n = snprintf(out, out_bytes, "denominators=%s; lattice=%s; cells=%s; gradient=%s%s", denom, lattice, cells,
-                         grad, mb ? " + multiblank_fixup_kernel" : "");
+                         grad, (mb && !gp.RT) ? " + multiblank_fixup_kernel" : "");
   return (n < 0 || (size_t)n >= out_bytes) ? MI_TRANSDUCER_INVALID_VALUE : MI_TRANSDUCER_SUCCESS;
 }
 

@@ -269,39 +269,6 @@ def export_lattice(workspace, act_lens, label_lens, B, T, U, num_durations=0):
     return denom, alphas, betas, llf, llb
 
 
-def set_lattice_mode(mode):
-    """0: per loss, whichever lattice kernel measured faster; 1: always the log-domain recursions; 2: the scaled
-    (probability-domain) recursions wherever the shape allows them.  Process-wide; for tests and A/B timing."""
-    _native.check_status(_native.lib().mi_transducer_set_lattice_mode(int(mode)), "set_lattice_mode")
-
-
-def lattice_formats(workspace, B, T, U, num_durations=0):
-    """int32[B]: per utterance, the format the last RNNT lattice kernel left in `workspace` (0 logs, 1 scaled)."""
-    off, per, word = ctypes.c_size_t(0), ctypes.c_int(0), ctypes.c_int(0)
-    status = _native.lib().mi_transducer_scale_segment(
-        B, T, U, num_durations, ctypes.byref(off), ctypes.byref(per), ctypes.byref(word)
-    )
-    _native.check_status(status, "scale_segment")
-    seg = workspace[off.value : off.value + 4 * per.value * B].view(torch.int32).view(B, per.value)
-    return seg[:, word.value].clone()
-
-
-def lattice_diagnostics(workspace, B, T, U):
-    """int32[B, 2] of the scaled RNNT lattice kernel: why an utterance took the log route (bit 0 an arc probability
-    out of range, bits 1 / 2 a direction ran out of range, bit 3 the exponent bound, bit 4 totals differ; 0 if it
-    did not), and the exponent spread it measured."""
-    off, per, word = ctypes.c_size_t(0), ctypes.c_int(0), ctypes.c_int(0)
-    status = _native.lib().mi_transducer_scale_segment(B, T, U, 0, ctypes.byref(off), ctypes.byref(per), ctypes.byref(word))
-    _native.check_status(status, "scale_segment")
-    seg = workspace[off.value : off.value + 4 * per.value * B].view(torch.int32).view(B, per.value)
-    return seg[:, 2:4].clone()
-
-
-def set_prefill_min_bytes(nbytes):
-    """Gradient tensors below this size get no riders in their lattice launch (process-wide; 32 MiB unless set)."""
-    _native.check_status(_native.lib().mi_transducer_set_prefill_min_bytes(int(nbytes)), "set_prefill_min_bytes")
-
-
 def prefilled_cells(workspace, act_lens, label_lens, B, T, U, row_elems, elem_bytes, num_durations=0):
     """bool[B, T, U]: the padded cells whose gradient rows the riders of the last forward call with prefill_grads
     zero-filled, read from the record in `workspace`.  row_elems = V + D of the gradient rows."""
@@ -380,10 +347,17 @@ def rnnt_loss_cpu(
     return True
 
 
+def _riders_code(riders):
+    """None: by the size of the gradient (32 MiB and more); True / False: with / without riders in the lattice launch."""
+    return _native.RIDERS_AUTO if riders is None else (_native.RIDERS_ON if riders else _native.RIDERS_OFF)
+
+
 def rnnt_loss_gpu(
-    acts, labels, input_lengths, label_lengths, costs, grads, blank_label, fastemit_lambda, clamp, num_threads=0
-):
-    """Drop-in for rnnt.py:138-236: costs (float32 [B]) and grads (or None) are filled in place."""
+    acts, labels, input_lengths, label_lengths, costs, grads, blank_label, fastemit_lambda, clamp, num_threads=0,
+    *, riders=None,
+):  # fmt: skip
+    """Drop-in for rnnt.py:138-236: costs (float32 [B]) and grads (or None) are filled in place.  `riders` (not in
+    the reference; same results either way): see _riders_code."""
     del num_threads  # an OpenMP knob of the reference's CPU path; unused on the GPU there too
     _require_gpu(acts, "rnnt_loss_gpu")
     B, T, U, V = acts.shape
@@ -394,7 +368,7 @@ def rnnt_loss_gpu(
         status = _native.lib().mi_rnnt_loss(
             _ptr(acts), _dtype_code(acts), _labels_ptr(labels), _ptr(input_lengths), _ptr(label_lengths), _ptr(costs),
             _ptr(grads), None, 0, 1.0, B, T, U, V, int(blank_label), float(fastemit_lambda), float(clamp),
-            _ptr(workspace), workspace.numel(), _stream(acts.device),
+            _riders_code(riders), _ptr(workspace), workspace.numel(), _stream(acts.device),
         )  # fmt: skip
     _native.check_status(status, "Could not calculate forward scores")
     # the caching allocator frees `workspace` in stream order, so it may go out of scope here
@@ -403,7 +377,7 @@ def rnnt_loss_gpu(
 
 def tdt_loss_gpu(
     label_acts, duration_acts, labels, input_lengths, label_lengths, costs, label_grads, duration_grads, blank_label,
-    durations, fastemit_lambda, clamp, num_threads, sigma, omega,
+    durations, fastemit_lambda, clamp, num_threads, sigma, omega, *, riders=None,
 ):  # fmt: skip
     """Drop-in for rnnt.py:239-363, argument for argument: label_acts [B,T,U,V] are raw token logits,
     duration_acts [B,T,U,D] duration log-probs; costs [B], label_grads [B,T,U,V] (gradient w.r.t. the token
@@ -432,7 +406,7 @@ def tdt_loss_gpu(
             _ptr(label_acts), _ptr(duration_acts), _dtype_code(label_acts), _labels_ptr(labels), _ptr(input_lengths),
             _ptr(label_lengths), _ptr(costs32), _ptr(label_grads), _ptr(duration_grads), None, 0, 1.0, B, T, U, V, D,
             dur_ptr, int(blank_label), float(fastemit_lambda), float(clamp), float(sigma), int(use_plain_rnnt),
-            _ptr(workspace), workspace.numel(), _stream(label_acts.device),
+            _riders_code(riders), _ptr(workspace), workspace.numel(), _stream(label_acts.device),
         )  # fmt: skip
     del keep
     _native.check_status(status, "Could not calculate forward scores")
@@ -441,7 +415,8 @@ def tdt_loss_gpu(
     return True
 
 
-def rnnt_loss_static(acts, labels, input_lengths, label_lengths, costs, grads, blank_label, fastemit_lambda, clamp):
+def rnnt_loss_static(acts, labels, input_lengths, label_lengths, costs, grads, blank_label, fastemit_lambda, clamp,
+                     *, riders=None):
     """rnnt_loss_gpu for callers that must not allocate (HIP graph capture, serving loops): same results, but the
     lattice state lives in a 64 MiB device array built into the library instead of a workspace tensor, so this
     function creates no tensor at all.  Shapes whose workspace is larger raise RuntimeError.  Calls on one GPU
@@ -454,7 +429,7 @@ def rnnt_loss_static(acts, labels, input_lengths, label_lengths, costs, grads, b
         status = _native.lib().mi_rnnt_loss_static(
             _ptr(acts), _dtype_code(acts), _labels_ptr(labels), _ptr(input_lengths), _ptr(label_lengths), _ptr(costs),
             _ptr(grads), None, 0, 1.0, B, T, U, V, int(blank_label), float(fastemit_lambda), float(clamp),
-            _stream(acts.device),
+            _riders_code(riders), _stream(acts.device),
         )  # fmt: skip
     _native.check_status(status, "rnnt_loss_static")
     return True
@@ -462,7 +437,7 @@ def rnnt_loss_static(acts, labels, input_lengths, label_lengths, costs, grads, b
 
 def combined_tdt_loss_gpu(
     acts, labels, input_lengths, label_lengths, costs, grads, blank_label, durations, fastemit_lambda, clamp,
-    num_threads=0, sigma=0.0, use_plain_rnnt=False,
+    num_threads=0, sigma=0.0, use_plain_rnnt=False, *, riders=None,
 ):  # fmt: skip
     """TDT on the COMBINED [B,T,U,V+D] logits (what TDTLossNumba.forward receives, rnnt_pytorch.py:554-583): the
     split, the duration log_softmax and its backward happen in the kernels, and grads is w.r.t. the combined
@@ -479,8 +454,8 @@ def combined_tdt_loss_gpu(
         status = _native.lib().mi_tdt_loss(
             _ptr(acts), _dtype_code(acts), _labels_ptr(labels), _ptr(input_lengths), _ptr(label_lengths), _ptr(costs),
             _ptr(grads), None, 0, 1.0, B, T, U, VD - D, D, dur_ptr, int(blank_label), float(fastemit_lambda),
-            float(clamp), float(sigma), int(bool(use_plain_rnnt)), _ptr(workspace), workspace.numel(),
-            _stream(acts.device),
+            float(clamp), float(sigma), int(bool(use_plain_rnnt)), _riders_code(riders), _ptr(workspace),
+            workspace.numel(), _stream(acts.device),
         )  # fmt: skip
     del keep
     _native.check_status(status, "Could not calculate forward scores")
@@ -489,7 +464,7 @@ def combined_tdt_loss_gpu(
 
 def multiblank_rnnt_loss_gpu(
     acts, labels, input_lengths, label_lengths, costs, grads, blank_label, big_blank_durations, fastemit_lambda, clamp,
-    num_threads=0, sigma=0.0,
+    num_threads=0, sigma=0.0, *, riders=None,
 ):  # fmt: skip
     """Multi-blank counterpart (rnnt.py:366-483): acts [B,T,U,V] with the big blanks at blank_label-1-i;
     costs is float32 [B], grads (or None) has the shape and dtype of acts."""
@@ -504,8 +479,8 @@ def multiblank_rnnt_loss_gpu(
         status = _native.lib().mi_multiblank_loss(
             _ptr(acts), _dtype_code(acts), _labels_ptr(labels), _ptr(input_lengths), _ptr(label_lengths), _ptr(costs),
             _ptr(grads), None, 0, 1.0, B, T, U, V, len(big_blank_durations), dur_ptr, int(blank_label),
-            float(fastemit_lambda), float(clamp), float(sigma), _ptr(workspace), workspace.numel(),
-            _stream(acts.device),
+            float(fastemit_lambda), float(clamp), float(sigma), _riders_code(riders), _ptr(workspace),
+            workspace.numel(), _stream(acts.device),
         )  # fmt: skip
     del keep
     _native.check_status(status, "Could not calculate forward scores")

@@ -15,8 +15,12 @@ What is done differently underneath:
     log-softmax happens inside the kernels.  CPU tensors go to the host library (RNNT
     only, as in the reference; TDT and multi-blank raise there as they do in the reference).
   * the gradient is computed in `backward`, by one kernel pass that already folds
-    in `grad_output`, the 'mean' reduction's 1/B, FastEmit and the clamp; forward
-    keeps a few MB of lattice state instead of a gradient tensor the size of `acts`.
+    in `grad_output`, the 'mean' reduction's 1/B, FastEmit and the clamp.  For logits
+    below 32 MiB forward keeps only a few MB of lattice state; from 32 MiB on (and when
+    acts requires a gradient) forward ALSO allocates the gradient tensor, the size of
+    `acts`, as the reference does (which computes the gradient there): the lattice launch
+    zero-fills its padded cells while it runs.  That tensor is held until backward runs or
+    the graph is dropped; MI_TRANSDUCER_PREFILL=0 in the environment restores the small footprint.
   * the shape-vs-lengths check reads both maxima back with one small copy that
     overlaps the forward kernels instead of two blocking torch.max calls.
 """
@@ -126,12 +130,15 @@ class _ValidatedLengths(threading.local):
     tensor's version on every in-place write), against the same shape cannot give another answer, so the read-back
     and the host wait it costs are skipped -- repeated calls on one batch (gradient accumulation, benchmarks) then
     never block the host.  Writes that bypass the version counter (`.data`, foreign kernels) are not seen; what is
-    lost then is only the ValueError for a malformed batch, the kernels clamp lengths anyway."""
+    lost then is only the ValueError for a malformed batch, the kernels clamp lengths anyway.
+    MI_TRANSDUCER_STRICT_LENGTH_CHECK=1 in the environment switches the memory off: every call then reads the maxima
+    back, as certify_inputs of the reference does (rnnt_pytorch.py:628-634)."""
 
     entry = None
 
 
 _validated = _ValidatedLengths()
+_STRICT_LENGTH_CHECK = os.environ.get("MI_TRANSDUCER_STRICT_LENGTH_CHECK", "") == "1"
 
 
 class _PendingLengthCheck:
@@ -145,7 +152,8 @@ class _PendingLengthCheck:
         self.tensors = (lengths, label_lengths)
         self.event = self.host = None
         seen = _validated.entry
-        if seen is not None and seen[0]() is lengths and seen[1]() is label_lengths and seen[2] == self.key:
+        if (not _STRICT_LENGTH_CHECK and seen is not None and seen[0]() is lengths and seen[1]() is label_lengths
+                and seen[2] == self.key):
             return  # these very tensors, unmodified, passed against this shape
         if lengths.is_cuda:
             # One small kernel on the auxiliary stream, ordered after whatever produced the lengths

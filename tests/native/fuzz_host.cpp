@@ -52,22 +52,16 @@ static void fuzz_plan(std::mt19937& rng, int iterations) {
     const bool want = B > 0 && T > 0 && U > 0 && D >= 0 && U <= MI_TRANSDUCER_MAX_U && D <= MI_TRANSDUCER_MAX_DURATIONS;
     EXPECT(ok == want, "B %d T %d U %d D %d", B, T, U, D);
     if (ok) {
-      const size_t offs[] = {L.off_denom, L.off_arcs,  L.off_alphas, L.off_betas, L.off_ll,
-                             L.off_coef,  L.off_scale, L.off_fill,   L.total};
-      for (int i = 0; i + 1 < 9; ++i) EXPECT(offs[i] < offs[i + 1] && (offs[i] & 255) == 0, "segment %d", i);
+      const size_t offs[] = {L.off_denom, L.off_arcs, L.off_alphas, L.off_betas, L.off_ll,
+                             L.off_coef,  L.off_fill, L.total};
+      for (int i = 0; i + 1 < 8; ++i) EXPECT(offs[i] < offs[i + 1] && (offs[i] & 255) == 0, "segment %d", i);
       EXPECT(L.Us >= U && L.Us == 64 * L.K && L.ND == T + U - 1 && L.A == 2 + D && L.CS >= kCoefBase + D, "layout");
       const size_t cells = (size_t)B * T * U, skew = (size_t)B * L.ND * L.Us;
       EXPECT(L.off_arcs - L.off_denom >= cells * 4 && L.off_alphas - L.off_arcs >= skew * L.A * 4 &&
                  L.off_betas - L.off_alphas >= skew * 8 && L.off_ll - L.off_betas >= skew * 8 &&
-                 L.off_coef - L.off_ll >= (size_t)B * 16 && L.off_scale - L.off_coef >= cells * L.CS * 4,
+                 L.off_coef - L.off_ll >= (size_t)B * 16 && L.off_fill - L.off_coef >= cells * L.CS * 4 &&
+                 L.total - L.off_fill >= (size_t)kFillInts * 4,
              "segment sizes B %d T %d U %d D %d", B, T, U, D);
-      // the scale segment: a 16-byte aligned header per utterance and an exponent pair for every block of diagonals,
-      // one block past the last diagonal included; the arc probabilities of the scaled RNNT lattice behind the rest
-      EXPECT(L.SG % 4 == 0 && L.SG >= kScaleHeader + 2 * (L.ND / kScaleBlock + 2) &&
-                 L.off_fill - L.off_scale >= (size_t)B * L.SG * 4 && L.total - L.off_fill >= (size_t)kFillInts * 4 &&
-                 L.off_arcp == L.total &&
-                 L.total_scaled - L.off_arcp >= (D == 0 ? skew * 16 : 0) && (L.off_arcp & 255) == 0,
-             "scale segment B %d T %d U %d D %d", B, T, U, D);
     }
     // rows per prefill item: a power of two up to eight, down to one for rows beyond 32 KB, never beyond 64 KB an item
     {

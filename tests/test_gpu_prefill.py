@@ -15,14 +15,8 @@ from gpu_utils import DEV
 
 pytestmark = pytest.mark.gpu
 
-
-
-@pytest.fixture(autouse=True)
-def riders_for_every_size():
-    rnnt.set_prefill_min_bytes(0)  # the shapes here are far below the size from which a forward call takes riders
-    yield
-    rnnt.set_prefill_min_bytes(32 << 20)
-
+# (a forward call that is handed a gradient buffer takes riders whatever the size of the problem: whether that pays is
+# the caller's decision -- the modules and the combined entry points decide by the size of the gradient)
 
 DURATIONS = [0, 1, 2, 3]
 BIG_BLANKS = [2, 4]
@@ -238,21 +232,56 @@ def test_replayed_from_a_graph(kind):
         assert said.any(), f"the riders did nothing on replay {replay}"
 
 
-def test_small_gradients_get_no_riders():
+def test_combined_entry_point_decides_by_size_unless_told():
+    """mi_rnnt_loss with riders = AUTO launches none for a gradient below 32 MiB (the record stays empty), ON fills
+    padding beside a lattice of several hundred anti-diagonals, OFF never does; the results are the same bits."""
+    import ctypes
+
     B, T, U, V = 4, 300, 40, 257
     acts, labels, al, ll = make(7, B, T, U, V, torch.float32)
     al[1], al[2] = 40, 150
-    rnnt.set_prefill_min_bytes(acts.numel() * 4 + 1)
-    c0, g0, _ = run("rnnt", acts, labels, al, ll, False)
-    c1, g1, after_forward = run("rnnt", acts, labels, al, ll, True)
-    assert torch.equal(c0, c1) and torch.equal(g0, g1) and torch.isnan(after_forward).all()
+    assert acts.numel() * 4 < (32 << 20)
+    stream = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+    out = {}
+    for riders in (_native.RIDERS_AUTO, _native.RIDERS_OFF, _native.RIDERS_ON):
+        ws = rnnt.new_workspace(acts)
+        ws.fill_(255)
+        costs = torch.empty(B, dtype=torch.float32, device=DEV)
+        grads = torch.full_like(acts, float("nan"))
+        st = _native.lib().mi_rnnt_loss(acts.data_ptr(), 0, labels.data_ptr(), al.data_ptr(), ll.data_ptr(),
+                                        costs.data_ptr(), grads.data_ptr(), None, 0, 1.0, B, T, U, V, V - 1, 0.01, 0.0,
+                                        riders, ws.data_ptr(), ws.numel(), stream)  # fmt: skip
+        assert st == _native.SUCCESS
+        torch.cuda.synchronize()
+        out[riders] = (costs, grads, rnnt.prefilled_cells(ws, al, ll, B, T, U, V, 4))
+    assert not out[_native.RIDERS_AUTO][2].any() and not out[_native.RIDERS_OFF][2].any()
+    assert out[_native.RIDERS_ON][2].any(), "riders = ON filled nothing beside a lattice of 340 anti-diagonals"
+    for riders in (_native.RIDERS_OFF, _native.RIDERS_ON):
+        assert torch.equal(out[riders][0], out[_native.RIDERS_AUTO][0])
+        assert torch.equal(out[riders][1], out[_native.RIDERS_AUTO][1])
+    assert torch.isfinite(out[_native.RIDERS_ON][1]).all()
+
+
+def test_riders_fill_something_at_the_benchmark_shape():
+    """B=16, T=375, U=121, V=1025 fp32 through the module: the riders of its lattice launch must fill part of the
+    padding -- a driver or firmware that parks every rider would otherwise only show as a slower step."""
+    cfg, acts, labels, al, ll = synthetic.make_inputs(1, device=DEV, generate_on_device=True)
+    assert rnnt_pytorch._prefill_wanted(acts)
+    ws = rnnt.new_workspace(acts)
+    costs = torch.empty(cfg.B, dtype=torch.float32, device=DEV)
+    grads = torch.empty_like(acts)
+    filled = []
+    for _ in range(3):
+        rnnt.rnnt_forward(acts, labels, al, ll, costs, cfg.blank, 0.0, True, ws, grads)
+        filled.append(int(rnnt.prefilled_cells(ws, al, ll, cfg.B, cfg.T, cfg.U, cfg.V, 4).sum()))
+    assert max(filled) > 0, filled
 
 
 @pytest.mark.parametrize("omega", [0.0, 1.0])
 def test_function_level_seams_take_riders_by_themselves(omega):
     """rnnt_loss_gpu / tdt_loss_gpu (the reference's signatures: split token logits and duration log-probs, also its
     plain-RNNT branch) / combined_tdt_loss_gpu / multiblank_rnnt_loss_gpu hand their gradient buffer to the lattice
-    launch on their own: with the size threshold at 0 and out of reach the results must be the same bits."""
+    launch on their own: with riders forced on and off the results must be the same bits."""
     B, T, U, V, D = 4, 200, 30, 130, len(DURATIONS)
     acts, labels, al, ll = make(13, B, T, U, V + D, torch.float32)
     al[1], al[2] = 30, 90
@@ -260,24 +289,26 @@ def test_function_level_seams_take_riders_by_themselves(omega):
     duration_acts = torch.log_softmax(acts[..., V:], dim=-1).contiguous()
     mb_acts = acts[..., : V + len(BIG_BLANKS)].contiguous()
     out = {}
-    for threshold in (0, 1 << 40):
-        rnnt.set_prefill_min_bytes(threshold)
+    for riders in (True, False):
         res = []
         costs, grads = torch.empty(B, device=DEV), torch.full_like(label_acts, float("nan"))
-        rnnt.rnnt_loss_gpu(label_acts, labels, al, ll, costs, grads, V - 1, 0.01, 0.0)
+        rnnt.rnnt_loss_gpu(label_acts, labels, al, ll, costs, grads, V - 1, 0.01, 0.0, riders=riders)
         res += [costs, grads]
         costs, lg, dg = torch.empty(B, device=DEV), torch.full_like(label_acts, float("nan")), torch.full_like(duration_acts, float("nan"))
-        rnnt.tdt_loss_gpu(label_acts, duration_acts, labels, al, ll, costs, lg, dg, V - 1, DURATIONS, 0.0, 0.0, 0, 0.05, omega)
+        rnnt.tdt_loss_gpu(label_acts, duration_acts, labels, al, ll, costs, lg, dg, V - 1, DURATIONS, 0.0, 0.0, 0, 0.05, omega,
+                          riders=riders)  # fmt: skip
         res += [costs, lg, dg]
         costs, grads = torch.empty(B, device=DEV), torch.full_like(acts, float("nan"))
-        rnnt.combined_tdt_loss_gpu(acts, labels, al, ll, costs, grads, V - 1, DURATIONS, 0.0, 0.0, 0, 0.05, omega > 0.5)
+        rnnt.combined_tdt_loss_gpu(acts, labels, al, ll, costs, grads, V - 1, DURATIONS, 0.0, 0.0, 0, 0.05, omega > 0.5,
+                                   riders=riders)  # fmt: skip
         res += [costs, grads]
         costs, grads = torch.empty(B, device=DEV), torch.full_like(mb_acts, float("nan"))
-        rnnt.multiblank_rnnt_loss_gpu(mb_acts, labels, al, ll, costs, grads, V + len(BIG_BLANKS) - 1, BIG_BLANKS, 0.0, 0.0, 0, 0.05)
+        rnnt.multiblank_rnnt_loss_gpu(mb_acts, labels, al, ll, costs, grads, V + len(BIG_BLANKS) - 1, BIG_BLANKS, 0.0, 0.0, 0,
+                                      0.05, riders=riders)  # fmt: skip
         res += [costs, grads]
         torch.cuda.synchronize()
-        out[threshold] = res
-    for a, b in zip(out[0], out[1 << 40]):
+        out[riders] = res
+    for a, b in zip(out[True], out[False]):
         assert torch.isfinite(a).all() and torch.equal(a, b)
 
 

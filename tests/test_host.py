@@ -82,7 +82,10 @@ def test_kernel_plan_of_the_documented_shapes(built_lib):
     # 257 whole vectors, one past a power of two: 5 vectors per lane in pass 1, a third (nearly empty) vector per
     # thread in the gradient pass rather than twice the threads
     assert p["denominators"] == "denom_rows_kernel<f32, R=5, RPW=1>"
-    assert p["gradient"] == "grad_block_kernel<f32, RT=128, NVT=3, coef> + multiblank_fixup_kernel"
+    # (that kernel writes the big blanks' entries itself; only the other gradient kernels are followed by a fix-up)
+    assert p["gradient"] == "grad_block_kernel<f32, RT=128, NVT=3, coef>"
+    p = plan(F32, 4, 50, 21, 32, num_big_blanks=3)  # short rows: the wave-per-row kernel, then the fix-up kernel
+    assert p["gradient"] == "grad_rows_kernel<f32, R=1, coef> + multiblank_fixup_kernel"
     p = plan(F32, 2, 50, 1024, 1028, max_duration=8, num_big_blanks=3)  # ring of 9 x 6 x 1024 doubles > 160 KB of LDS
     assert p["lattice"] == "multiblank_lattice_pull_kernel"
     p = plan(F32, 2, 50, 513, 1025, D=9, max_duration=8)  # beyond 256 label columns: a wave per direction
