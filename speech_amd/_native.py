@@ -35,6 +35,9 @@ HIPCC_FLAGS = [
     "-shared",
     # keep the compiler from forming packed-fp32 instructions
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+    # the first dwords of a kernel's arguments arrive in scalar registers with the wave instead of being fetched by
+    # its first instructions (the kernels order their arguments for it)
+    "-mllvm", "-amdgpu-kernarg-preload-count=16",
 ]  # fmt: skip
 
 

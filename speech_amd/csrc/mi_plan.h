@@ -87,14 +87,16 @@ inline FastDiv make_fastdiv(unsigned d) {
   f.shift = l;
   return f;
 }
+// the two divisions that split a workgroup id into (b, t, chunk), in three words (the shifts share one): this block
+// is among the kernel arguments that arrive in registers with the wave, where every word counts
 struct GridDiv {
-  FastDiv chunks, T;
+  unsigned mul_chunks, mul_T, shifts;  // shifts = shift of the division by nchunks | shift of the division by T << 8
 };
+inline FastDiv griddiv_chunks(const GridDiv& g) { return FastDiv{g.mul_chunks, g.shifts & 255u}; }
+inline FastDiv griddiv_frames(const GridDiv& g) { return FastDiv{g.mul_T, g.shifts >> 8}; }
 inline GridDiv make_griddiv(int nchunks, int T) {
-  GridDiv g;
-  g.chunks = make_fastdiv((unsigned)nchunks);
-  g.T = make_fastdiv((unsigned)T);
-  return g;
+  const FastDiv c = make_fastdiv((unsigned)nchunks), t = make_fastdiv((unsigned)T);
+  return GridDiv{c.mul, t.mul, c.shift | (t.shift << 8)};
 }
 
 

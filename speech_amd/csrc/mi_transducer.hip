@@ -38,10 +38,10 @@
 #define MI_XCD_MAP 1  // 1: each XCD streams one contiguous eighth of the (b,t) rows
 #endif
 #ifndef MI_NT_K1
-#define MI_NT_K1 0    // non-temporal loads in the long-row denominator pass
+#define MI_NT_K1 1    // non-temporal loads in the denominator pass
 #endif
 #ifndef MI_NT_K4
-#define MI_NT_K4 0    // non-temporal loads in the long-row gradient pass
+#define MI_NT_K4 1    // non-temporal loads in the gradient pass
 #endif
 
 namespace {

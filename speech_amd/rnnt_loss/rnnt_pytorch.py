@@ -72,14 +72,16 @@ def _aux_stream(device):
 
 def grads_like(acts):
     """An uninitialised tensor of the shape and dtype of acts whose storage starts at the same offset within a
-    16-byte line as acts does.  The gradient pass stores whole 16-byte vectors where the logits row has them, which
-    needs the two buffers in phase; a fresh allocation is 16-byte aligned, a view such as `big[1:]` need not be."""
-    phase = acts.data_ptr() & 15
+    256-byte block as acts does.  The gradient pass stores whole 16-byte vectors where the logits row has them, which
+    needs the two buffers in phase, and its stores stream when each instruction covers whole 64-byte pieces, which
+    they do when the phases agree that far; a fresh allocation is 256-byte aligned, a view such as `big[1:]` need
+    not be."""
+    phase = acts.data_ptr() & 255
     if phase == 0:
         return torch.empty_like(acts)
     size = acts.element_size()
-    flat = torch.empty(acts.numel() + 16 // size, dtype=acts.dtype, device=acts.device)
-    first = ((phase - flat.data_ptr()) & 15) // size
+    flat = torch.empty(acts.numel() + 256 // size, dtype=acts.dtype, device=acts.device)
+    first = ((phase - flat.data_ptr()) & 255) // size
     return flat[first : first + acts.numel()].view(acts.shape)
 
 

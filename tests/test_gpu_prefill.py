@@ -237,7 +237,7 @@ def test_combined_entry_point_decides_by_size_unless_told():
     padding beside a lattice of several hundred anti-diagonals, OFF never does; the results are the same bits."""
     import ctypes
 
-    B, T, U, V = 4, 300, 40, 257
+    B, T, U, V = 4, 300, 40, 129
     acts, labels, al, ll = make(7, B, T, U, V, torch.float32)
     al[1], al[2] = 40, 150
     assert acts.numel() * 4 < (32 << 20)
