@@ -46,8 +46,13 @@ HBM_PEAK_GBPS = 8000.0  # MI355X HBM3E, published peak
 # this script, scaled by what the same counters read for mi_transducer_copy_probe of known size
 # (summaries under profiles/).  None = not measured for that workload.
 MEASURED_TRAFFIC_KIB = {
-    # workload: (FETCH_SIZE, WRITE_SIZE) of the gradient-pass kernel in KiB per dispatch, and the factors the same
-    # counters need to read a 1 GiB copy right (profiles/transducer_kernels_<cfg>_hbm_traffic.md)
+    # workload: (FETCH_SIZE, WRITE_SIZE) of the gradient-pass kernel in KiB per dispatch; the factors below are what the
+    # same counters need to read a 1 GiB copy right (profiles/transducer_kernels_<cfg>_hbm_traffic.md)
+    "cfg2_rnnt_B16_T375_U121_V1025_f32": (810650, 2597095),
+    "cfg3_rnnt_B32_T750_U201_V1025_bf16": (3005433, 8598631),
+    "cfg4_tdt_B16_T375_U121_V1025_D5_f32": (760668, 1754402),
+    "cfg5_rnnt_B8_T250_U101_V16385_f32": (3670722, 12821044),
+    "cfg6_multiblank_B16_T375_U121_V1028_f32": (684935, 1990962),
 }
 TRAFFIC_SCALE = (2.0, 1.0)
 
@@ -71,6 +76,9 @@ def parse_args():
     ap.add_argument("--same-tensors", action="store_true",
                     help="headline loop over ONE set of tensors (the length check is then remembered and pass 1 starts "
                          "in the last step's cache tail); default: fresh length tensors and alternating logits buffers")
+    ap.add_argument("--full-lengths", action="store_true",
+                    help="every utterance at full length (act_lens = T, label_lens = U-1): the same kernels without "
+                         "padding, for counter profiles that hold ragged against full lengths")
     ap.add_argument("--cpu-sample-utterances", type=int, default=16)
     return ap.parse_args()
 
@@ -457,6 +465,9 @@ def main():
     _native.lib()  # fail now if the HIP library is missing
 
     cfg, acts, labels, act_lens, label_lens = synthetic.make_inputs(args.workload, device=dev, generate_on_device=True)
+    if args.full_lengths:
+        act_lens.fill_(cfg.T)
+        label_lens.fill_(cfg.U - 1)
     if args.op == "joint":
         del acts
         return run_joint(args, torch, dev, cfg, labels, act_lens, label_lens)
@@ -569,7 +580,7 @@ def main():
         "dtype": {torch.float32: "f32", torch.bfloat16: "bf16", torch.float16: "f16"}[cfg.dtype],
         "data": "synthetic",
         "config": {
-            "workload": cfg.name + ("_logprobs" if logprobs else ""),
+            "workload": cfg.name + ("_logprobs" if logprobs else "") + ("_full_lengths" if args.full_lengths else ""),
             "B": cfg.B, "T": cfg.T, "U": cfg.U, "V": cfg.V, "D": cfg.D,
             "valid_cells": nbytes["c_valid"], "cells": nbytes["cells"],
             "fastemit_lambda": cfg.fastemit_lambda, "clamp": cfg.clamp, "sigma": cfg.sigma,

@@ -16,20 +16,27 @@ How each function is pinned (tests/test_oracle_*.py):
   tdt_*             reference fixed vector (cost 4.155739 + 42 grads),
                     brute-force (token,duration) path enumeration,
                     torch autograd, T=1 and U=1 closed forms ......... pinned
-  tdt_* FastEmit    PARITY UNPINNED: no reference vector or test exists for
-                    TDT with fastemit_lambda > 0; the terms are derived
-                    from gpu_rnnt_kernel.py:1353-1437 and checked only
-                    against their meaning (label-arc log-prob gradient
-                    x (1+lambda) through the token softmax Jacobian, the
-                    duration branch untouched) in torch autograd ..... derived
+  tdt_* FastEmit    no reference vector or test exists for TDT with
+                    fastemit_lambda > 0; pinned by what the kernel's terms
+                    (gpu_rnnt_kernel.py:1353-1437) mean: the gradient of the
+                    label arcs' log-probs x (1+lambda) through the token
+                    softmax Jacobian, the duration branch untouched --
+                    tests/helpers.py differentiates exactly that with torch
+                    autograd, independently of the restated terms, and
+                    test_oracle_tdt.py::test_fastemit_by_definition holds the
+                    restatement to it at 1e-10 (a dropped sigma, a wrong beta
+                    index or FastEmit leaking into the durations fails it)
+                    .............................................. pinned
   multiblank_*      the reference holds no vector (its test compares two of
                     its own implementations on random input); with no big
                     blank and sigma = 0 it must give the RNNT golden vectors,
                     brute-force enumeration of every (token, blank-duration)
                     path, torch autograd of an alpha-only recursion,
                     llForward == beta(0,0) ........................... pinned
-  multiblank_* FastEmit  PARITY UNPINNED: derived only (gpu_rnnt_kernel.py:
-                    727-885), checked as for TDT
+  multiblank_* FastEmit  likewise no reference vector; pinned by the
+                    meaning of gpu_rnnt_kernel.py:727-885 (label-arc gradient
+                    x (1+lambda), blank and big-blank arcs untouched), as
+                    for TDT (tests/test_oracle_multiblank.py) ......... pinned
   joint_rnnt_loss   torch autograd (float64) through relu, linear and an
                     alpha-only recursion, with the bf16 roundings applied
                     straight-through; the loss part is rnnt_loss above;

@@ -6,6 +6,7 @@ import torch
 
 import oracle
 from speech_amd import MultiblankRNNTLossNumba, RNNTLossNumba, multiblank_rnnt_loss_gpu
+from speech_amd.rnnt_loss import rnnt
 
 from gpu_utils import DEV, call_loss, make_lengths, to_dev
 from helpers import multiblank_autograd
@@ -92,6 +93,47 @@ def test_label_axes_whose_ring_exceeds_lds(U, durs):
     labels = rng.randint(0, V - 1 - len(durs), size=(B, U - 1))
     # hundreds of log-sum-exp steps of up to ten terms: float rounding of the gradients reaches 5e-6 (the bar is 1e-4)
     check_against_oracle(acts, labels, np.array([T, 14]), np.array([U - 1, (U - 1) // 2]), V - 1, durs, 0.05, grad_atol=1e-5)
+
+
+@pytest.mark.parametrize(
+    "shape,durs,lens",
+    [
+        ((1, 15, 11, 6), [2, 3, 4], None),          # utils/test_gpu_rnnt_kernel.py:711-797 (alphas) and :800-886 (betas)
+        ((3, 40, 17, 12), [2, 4, 8], "ragged"),     # ragged lengths, a blank longer than some utterances' remainders
+        ((2, 23, 300, 15), [2, 3, 4, 5, 6, 7, 8, 9], "ragged"),  # the ring exceeds LDS: the kernel that pulls from memory
+    ],
+)
+def test_stage_level_lattice(shape, durs, lens):
+    """The forward variables, the backward variables and both log-likelihoods on their own, read out of the workspace
+    after the forward call (the reference tests its multi-blank alpha and beta kernels on their own too): an error
+    in alpha or beta that cancels in the gradient would not show in the end-to-end tests."""
+    B, T, U, V = shape
+    rng = np.random.RandomState(U + len(durs))
+    x = rng.randn(B, T, U, V).astype(np.float32)
+    labels = rng.randint(0, V - 1 - len(durs), size=(B, U - 1))
+    if lens is None:
+        act_lens, label_lens = [T] * B, [U - 1] * B
+    else:
+        act_lens, label_lens = make_lengths(rng, B, T, U, 3, 0)
+    acts = torch.tensor(x, device=DEV)
+    lab, al, ll = to_dev(labels, act_lens, label_lens)
+    costs = torch.empty(B, dtype=torch.float32, device=DEV)
+    ws = rnnt.new_workspace(acts, len(durs))
+    rnnt.multiblank_forward(acts, lab, al, ll, costs, V - 1, durs, 0.0, 0.05, True, ws)
+    denom, alphas, betas, llf, llb = [t.cpu().numpy() for t in rnnt.export_lattice(ws, al, ll, B, T, U, len(durs))]
+    c_ref, _, ex = oracle.multiblank_loss(x, labels, act_lens, label_lens, V - 1, durs, 0.05, want_grads=False)
+    valid = (np.arange(T)[None, :, None] < np.asarray(act_lens)[:, None, None]) & (
+        np.arange(U)[None, None, :] <= np.asarray(label_lens)[:, None, None]
+    )
+    assert np.abs(denom - ex["denom"])[valid].max() < 1e-5
+    # (cells no alignment reaches hold -inf in the oracle and the kernels' large negative stand-in here: compare
+    # the reachable ones, and require the others to be far below any reachable value)
+    for got, want in ((alphas, ex["alphas"]), (betas, ex["betas"])):
+        reach = valid & np.isfinite(want)
+        assert reach.any() and np.abs(got - want)[reach].max() < 2e-4 * max(1.0, np.abs(want[reach]).max() / 50)
+        assert np.all(got[valid & ~np.isfinite(want)] < want[reach].min() - 100)
+    assert np.allclose(llf, ex["ll_forward"], rtol=1e-6, atol=1e-5) and np.allclose(llb, llf, rtol=1e-6, atol=1e-5)
+    assert np.allclose(costs.cpu().numpy(), c_ref, rtol=1e-6)
 
 
 def test_blank_in_the_middle_and_reductions_and_half_precision():
