@@ -287,63 +287,75 @@ int mi_rnnt_logprobs_backward(const void* logits, int act_dtype, const int64_t* 
  * Every mi_joint_* call on a workspace takes the same D and num_big_blanks (both 0 for RNNT, at most one of them
  * non-zero): they are part of the workspace layout. */
 int mi_joint_workspace_bytes(int B, int T, int U, int H, int V, int D, int num_big_blanks, size_t* out_bytes);
+/* A forward call that a backward call is to follow keeps two things, a row per lattice cell in the kernel's tile
+ * order -- utterance by utterance, cell t*U_b + u, each utterance padded to a multiple of 128 rows:
+ *   saved_logits [saved_tiles*128][padded_vocabulary(V + D)] fp16: the logits (10 mantissa bits: the probabilities
+ *     the backward forms from them are as exact as the bf16 gradient entries they are rounded to);
+ *   saved_acts   [saved_tiles*128][H+16] bf16: the hidden activations (after activation and dropout) followed by
+ *     1, 1 and zeros, so that column H of dlogits^T . saved_acts is the gradient of the bias; zero rows past an
+ *     utterance's end.
+ * Both NULL: nothing is kept (inference).  saved_tiles must be at least mi_joint_tile_bound(B, T, U), the number of
+ * tiles of lattices without padding -- a bound known without reading the lengths back from the device; the tiles
+ * actually used (device int32 *tile_count, nullable) come first. */
+int mi_joint_tile_bound(int B, int T, int U); /* 0: no such lattice, or more tiles than the kernels index */
 int mi_joint_rnnt_forward(const void* f, const void* g, const void* weight, const void* bias, int weight_dtype,
                           const int64_t* labels, const int64_t* act_lens, const int64_t* label_lens, float* costs,
                           int* tile_count, float dropout_p, unsigned long long dropout_seed, int activation, int B, int T, int U, int H,
-                          int V, int blank, float fastemit_lambda, int with_betas, void* workspace,
-                          size_t workspace_bytes, void* stream);
+                          int V, int blank, float fastemit_lambda, int with_betas, void* saved_logits,
+                          void* saved_acts, long long saved_tiles, void* workspace, size_t workspace_bytes, void* stream);
 int mi_joint_tdt_forward(const void* f, const void* g, const void* weight, const void* bias, int weight_dtype,
                          const int64_t* labels, const int64_t* act_lens, const int64_t* label_lens, float* costs,
                          int* tile_count, float dropout_p, unsigned long long dropout_seed, int activation, int B, int T, int U, int H,
                          int V, int D, const int32_t* durations_host, int blank, float fastemit_lambda, float sigma,
-                         int with_betas, void* workspace, size_t workspace_bytes, void* stream);
+                         int with_betas, void* saved_logits, void* saved_acts, long long saved_tiles, void* workspace,
+                         size_t workspace_bytes, void* stream);
 int mi_joint_multiblank_forward(const void* f, const void* g, const void* weight, const void* bias, int weight_dtype,
                                 const int64_t* labels, const int64_t* act_lens, const int64_t* label_lens, float* costs,
                                 int* tile_count, float dropout_p, unsigned long long dropout_seed, int activation, int B, int T, int U,
                                 int H, int V, int num_big_blanks, const int32_t* big_blank_durations_host, int blank,
-                                float fastemit_lambda, float sigma, int with_betas, void* workspace,
-                                size_t workspace_bytes, void* stream);
+                                float fastemit_lambda, float sigma, int with_betas, void* saved_logits,
+                                void* saved_acts, long long saved_tiles, void* workspace, size_t workspace_bytes,
+                                void* stream);
 int mi_joint_dropout_mask(unsigned char* mask, float dropout_p, unsigned long long dropout_seed, int B, int T, int U,
                           int H, void* stream);
 
-/* Backward of the fused joint, first half: the logits are recomputed tile by tile exactly as in the forward call
- * (same dropout_p and dropout_seed) and turned into their gradient (gpu_rnnt_kernel.py:340-403 with grad_scale
- * folded in, as mi_rnnt_backward), which is stored as bf16 for the two matrix products that finish the job:
- *   d weight = dlogits^T . hidden   and   d hidden = dlogits . weight.
- * dlogits [rows][padded_vocabulary(V)] bf16: one row per lattice cell in the kernel's tile order -- utterance by
- *   utterance, cell t*U_b + u, each utterance padded to a multiple of 128 rows with zero rows; columns beyond V zero.
- * hidden [rows][H+16] bf16: the joint's hidden activations of the same rows (after ReLU and dropout) followed by
- *   1, 1 and zeros, so that column H of dlogits^T . hidden is the gradient of the bias.
- * `tiles` is the number of 128-row tiles the two buffers hold: at least what mi_joint_rnnt_forward wrote to
- * tile_count (device int32, nullable there), whose workspace this call needs unchanged (forward with
- * with_betas != 0).
- * TDT: dlogits has padded_vocabulary(V + D) columns, columns V .. V+D-1 the gradient of the duration logits
- * (gpu_rnnt_kernel.py:1244-1439 followed by the log_softmax backward); no clamp on those, as in the reference. */
+/* Backward of the fused joint (replaces autograd through the joint's Linear and the loss, modules/rnnt.py:1707-1724
+ * and gpu_rnnt_kernel.py:340-403).  The gradient of the logits (grad_scale folded in as in mi_rnnt_backward; rows past
+ * an utterance's end and columns beyond the vocabulary zero) is formed from the saved logits inside two kernels and
+ * never written out:
+ *   d_hidden [tiles*128][H] bf16 = dlogits . weight (rows as saved_logits; nullable: not wanted),
+ *   dw_part [slices][padded_vocabulary][H] float32, db_part [slices][padded_vocabulary] float32: partial sums of
+ *     d weight = dlogits^T . saved_acts and d bias = column sums of dlogits, one per slice of the rows; the caller adds
+ *     the slices up (both nullable together: not wanted).  A good `slices` is 256 / (padded_vocabulary / 128).
+ * `tiles`: the rows/128 that the buffers hold (the bound given to the forward call).  The workspace is the forward
+ * call's, unchanged (forward with with_betas != 0); saved_logits and saved_acts are only read.  Nothing is read back to
+ * the host and nothing is allocated.
+ * TDT: columns V .. V+D-1 of dlogits are the gradient of the duration logits (gpu_rnnt_kernel.py:1244-1439 followed
+ * by the log_softmax backward); no clamp on those, as in the reference. */
 int mi_joint_padded_vocabulary(int V);
-int mi_joint_rnnt_backward_logits(const void* f, const void* g, const int64_t* labels, const int64_t* act_lens,
-                                  const int64_t* label_lens, void* dlogits, void* hidden, int tiles,
-                                  const float* grad_scale, int grad_scale_stride,
-                                  float grad_mul, float dropout_p, unsigned long long dropout_seed, int activation, int B, int T, int U,
-                                  int H, int V, int blank, float fastemit_lambda, float clamp, void* workspace,
-                                  size_t workspace_bytes, void* stream);
-int mi_joint_tdt_backward_logits(const void* f, const void* g, const int64_t* labels, const int64_t* act_lens,
-                                 const int64_t* label_lens, void* dlogits, void* hidden, int tiles,
-                                 const float* grad_scale, int grad_scale_stride, float grad_mul, float dropout_p,
-                                 unsigned long long dropout_seed, int activation, int B, int T, int U, int H, int V, int D,
-                                 const int32_t* durations_host, int blank, float fastemit_lambda, float clamp,
-                                 float sigma, void* workspace, size_t workspace_bytes, void* stream);
-int mi_joint_multiblank_backward_logits(const void* f, const void* g, const int64_t* labels, const int64_t* act_lens,
-                                        const int64_t* label_lens, void* dlogits, void* hidden, int tiles,
-                                        const float* grad_scale, int grad_scale_stride, float grad_mul,
-                                        float dropout_p, unsigned long long dropout_seed, int activation, int B, int T, int U, int H,
-                                        int V, int num_big_blanks, const int32_t* big_blank_durations_host, int blank,
-                                        float fastemit_lambda, float clamp, float sigma, void* workspace,
-                                        size_t workspace_bytes, void* stream);
+int mi_joint_rnnt_backward(const int64_t* labels, const int64_t* act_lens, const int64_t* label_lens,
+                           void* saved_logits, const void* saved_acts, void* d_hidden, float* dw_part, float* db_part,
+                           int slices, long long tiles, const float* grad_scale, int grad_scale_stride, float grad_mul,
+                           int B, int T, int U, int H, int V, int blank, float fastemit_lambda, float clamp,
+                           void* workspace, size_t workspace_bytes, void* stream);
+int mi_joint_tdt_backward(const int64_t* labels, const int64_t* act_lens, const int64_t* label_lens,
+                          void* saved_logits, const void* saved_acts, void* d_hidden, float* dw_part, float* db_part,
+                          int slices, long long tiles, const float* grad_scale, int grad_scale_stride, float grad_mul,
+                          int B, int T, int U, int H, int V, int D, const int32_t* durations_host, int blank,
+                          float fastemit_lambda, float clamp, float sigma, void* workspace, size_t workspace_bytes,
+                          void* stream);
+int mi_joint_multiblank_backward(const int64_t* labels, const int64_t* act_lens, const int64_t* label_lens,
+                                 void* saved_logits, const void* saved_acts, void* d_hidden, float* dw_part,
+                                 float* db_part, int slices, long long tiles, const float* grad_scale,
+                                 int grad_scale_stride, float grad_mul, int B, int T, int U, int H, int V,
+                                 int num_big_blanks, const int32_t* big_blank_durations_host, int blank,
+                                 float fastemit_lambda, float clamp, float sigma, void* workspace,
+                                 size_t workspace_bytes, void* stream);
 
 /* Backward of the fused joint, last step: d_hidden [rows][H] bf16 (= dlogits . weight, rows as above) times the
  * activation's derivative, summed over u into d_f [B,T,H] and over t into d_g [B,U,H] (float32; either may be NULL; frames
  * and label positions outside an utterance get zeros).  The derivative is recomputed from f and g (the forward
- * call's bf16 inputs), `tiles` is the same count as in mi_joint_rnnt_backward_logits, the workspace the forward
+ * call's bf16 inputs), `tiles` is the same count as in mi_joint_rnnt_backward, the workspace the forward
  * call's. */
 int mi_joint_reduce_hidden(const void* d_hidden, const void* f, const void* g, const int64_t* act_lens,
                            const int64_t* label_lens, float* d_f, float* d_g, int tiles, float dropout_p,

@@ -21,7 +21,7 @@ CPU_SOURCES = [os.path.join(CSRC_DIR, "mi_cpu.cpp")]
 CPU_ABI_VERSION = 1
 CXX_FLAGS = ["-O3", "-std=c++17", "-fPIC", "-shared", "-fopenmp", "-Wall", "-Wextra"]
 
-ABI_VERSION = 18
+ABI_VERSION = 19
 SUCCESS, INVALID_VALUE, LAUNCH_FAILURE, TOO_LARGE = 0, 1, 2, 3
 STATIC_WORKSPACE_BYTES = 64 << 20
 DTYPE_F32, DTYPE_BF16, DTYPE_F16 = 0, 1, 2
@@ -111,25 +111,26 @@ _SIGNATURES = {
     "mi_rnnt_logprobs_backward": [_vp, _c_int, _vp, _vp, _vp, _vp, _vp, _vp, _c_int, _c_int, _c_int, _c_int, _c_int,
                                   _c_int, _vp, _c_size_t, _vp],
     "mi_joint_workspace_bytes": [_c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, ctypes.POINTER(_c_size_t)],
+    "mi_joint_tile_bound": [_c_int, _c_int, _c_int],
     "mi_joint_rnnt_forward": [_vp, _vp, _vp, _vp, _c_int, _vp, _vp, _vp, _vp, _vp, _c_float, ctypes.c_uint64, _c_int,
-                              _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_float, _c_int, _vp, _c_size_t, _vp],
+                              _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_float, _c_int, _vp, _vp,
+                              ctypes.c_longlong, _vp, _c_size_t, _vp],
     "mi_joint_tdt_forward": [_vp, _vp, _vp, _vp, _c_int, _vp, _vp, _vp, _vp, _vp, _c_float, ctypes.c_uint64, _c_int,
                              _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _vp, _c_int, _c_float, _c_float, _c_int, _vp,
-                             _c_size_t, _vp],
+                             _vp, ctypes.c_longlong, _vp, _c_size_t, _vp],
     "mi_joint_multiblank_forward": [_vp, _vp, _vp, _vp, _c_int, _vp, _vp, _vp, _vp, _vp, _c_float, ctypes.c_uint64,
                                     _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _vp, _c_int, _c_float, _c_float,
-                                    _c_int, _vp, _c_size_t, _vp],
+                                    _c_int, _vp, _vp, ctypes.c_longlong, _vp, _c_size_t, _vp],
     "mi_joint_dropout_mask": [_vp, _c_float, ctypes.c_uint64, _c_int, _c_int, _c_int, _c_int, _vp],
     "mi_joint_padded_vocabulary": [_c_int],
-    "mi_joint_rnnt_backward_logits": [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _c_int, _vp, _c_int, _c_float,
-                                      _c_float, ctypes.c_uint64, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int,
-                                      _c_float, _c_float, _vp, _c_size_t, _vp],
-    "mi_joint_tdt_backward_logits": [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _c_int, _vp, _c_int, _c_float,
-                                     _c_float, ctypes.c_uint64, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _vp,
-                                     _c_int, _c_float, _c_float, _c_float, _vp, _c_size_t, _vp],
-    "mi_joint_multiblank_backward_logits": [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _c_int, _vp, _c_int, _c_float,
-                                            _c_float, ctypes.c_uint64, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int,
-                                            _vp, _c_int, _c_float, _c_float, _c_float, _vp, _c_size_t, _vp],
+    "mi_joint_rnnt_backward": [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _c_int, ctypes.c_longlong, _vp, _c_int, _c_float,
+                               _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_float, _c_float, _vp, _c_size_t, _vp],
+    "mi_joint_tdt_backward": [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _c_int, ctypes.c_longlong, _vp, _c_int, _c_float,
+                              _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _vp, _c_int, _c_float, _c_float, _c_float,
+                              _vp, _c_size_t, _vp],
+    "mi_joint_multiblank_backward": [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _c_int, ctypes.c_longlong, _vp, _c_int,
+                                     _c_float, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _vp, _c_int, _c_float,
+                                     _c_float, _c_float, _vp, _c_size_t, _vp],
     "mi_joint_reduce_hidden": [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _c_int, _c_float, ctypes.c_uint64, _c_int, _c_int, _c_int,
                                _c_int, _c_int, _c_int, _c_int, _c_int, _vp, _c_size_t, _vp],
     "mi_joint_packed_weights": [_vp, _c_size_t, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int,
