@@ -400,12 +400,13 @@ int mi_transducer_length_maxima(const int64_t* act_lens, const int64_t* label_le
  * class.  The recording state is the library's only process-wide mutable state; it is guarded by a mutex, so the
  * calls are safe from any thread, but launches from several threads are then counted into the same classes.  Leave
  * it disabled outside benchmarks (disabled, a launch only reads one flag). */
-#define MI_PROFILE_DENOM 0   /* denom_rows_kernel / denom_block_kernel / denom_gather_kernel */
+#define MI_PROFILE_DENOM 0   /* denom_rows_kernel / denom_block_kernel / denom_gather_kernel / joint_lse_kernel */
 #define MI_PROFILE_LATTICE 1 /* rnnt_lattice_kernel / tdt_lattice_pair_kernel / tdt_lattice_kernel */
 #define MI_PROFILE_CELL 2    /* rnnt_cell_kernel / tdt_cell_kernel */
-#define MI_PROFILE_GRAD 3    /* grad_rows_kernel / grad_block_kernel / grad_stream_kernel */
+#define MI_PROFILE_GRAD 3    /* grad_rows_kernel / grad_block_kernel / grad_stream_kernel / joint_dhidden_kernel */
 #define MI_PROFILE_ZERO 4    /* zero_padding_kernel */
-#define MI_PROFILE_KERNELS 5
+#define MI_PROFILE_DWEIGHT 5 /* joint_dweight_kernel */
+#define MI_PROFILE_KERNELS 6
 int mi_transducer_profile_enable(int max_launches, unsigned kernel_mask);
 int mi_transducer_profile_read(int kernel_id, float* total_ms, int* launches);
 int mi_transducer_profile_disable(void);

@@ -250,6 +250,7 @@ PROFILE_KERNELS = {
     "cells": 2,
     "gradient_pass": 3,
     "zero_padding": 4,
+    "weight_gradient": 5,
 }
 
 
