@@ -397,11 +397,14 @@ def run_joint(args, torch, dev, cfg, labels, act_lens, label_lens):
         step()
     torch.cuda.synchronize()
     # the timed steps carry no events; the kernels' own times come from a second pass with the library's event pairs
+    torch.cuda.reset_peak_memory_stats(dev)
+    base_bytes = torch.cuda.memory_allocated(dev)
     t0 = time.perf_counter()
     for _ in range(args.steps):
         costs = step()
     torch.cuda.synchronize()
     wall = time.perf_counter() - t0
+    step_peak_bytes = torch.cuda.max_memory_allocated(dev) - base_bytes  # what a step allocates on top of its inputs
     _native.profile_enable(args.steps, ["denominator_pass", "lattice", "cells", "gradient_pass", "weight_gradient"])
     for _ in range(args.steps):
         step()
@@ -439,6 +442,7 @@ def run_joint(args, torch, dev, cfg, labels, act_lens, label_lens):
         "product_kernels": products,
         "whole_job": {"useful_tflop_per_step": 3 * flops / 1e12,
                       "achieved_tflops": 3 * flops / (ms_per_step * 1e-3) / 1e12,
+                      "step_peak_memory_GB": step_peak_bytes / 1e9,
                       "note": "three products per step (logits, d hidden, d weight), each in a kernel of this library; "
                               "no library GEMM and no host wait in the step"},
     }  # fmt: skip
