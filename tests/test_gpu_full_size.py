@@ -130,3 +130,60 @@ def test_full_size_configuration_1_against_the_whole_oracle():
                                         label_lens.cpu().numpy(), cfg.blank, dtype=np.float32)  # fmt: skip
     assert np.allclose(costs.detach().cpu().numpy(), c_cpu, rtol=COST_RTOL)
     assert np.abs(acts.grad.cpu().numpy() - g_cpu).max() < GRAD_ATOL
+
+
+def test_full_size_fused_joint():
+    """The fused joint + loss at the benchmark's lattice shape (cfg 2: B=16, T=375, U=121, V=1025) with H=640: 3070
+    tiles over 252 d-weight workgroups.  Checked (1) against the oracle on the smallest utterance cut out of the batch
+    (costs; d f and d g rows of that utterance), and (2) through properties that hold at any size: d bias sums to
+    zero over the vocabulary (every cell's gradient of the logits does), frames and label positions outside an
+    utterance get exactly nothing, the gradients are linear in grad_output, and sub-batches of four utterances give the
+    same costs bit for bit and the same gradients up to the rounding of their partial sums."""
+    from speech_amd.joint import joint_rnnt_loss
+
+    cfg, acts, labels, act_lens, label_lens = synthetic.make_inputs(1, device=DEV, generate_on_device=True)
+    del acts
+    B, T, U, V, H = cfg.B, cfg.T, cfg.U, cfg.V, 640
+    gen = torch.Generator(device=DEV).manual_seed(77)
+    f0 = torch.randn(B, T, H, device=DEV, generator=gen).to(torch.bfloat16)
+    g0 = torch.randn(B, U, H, device=DEV, generator=gen).to(torch.bfloat16)
+    W0 = torch.randn(V, H, device=DEV, generator=gen) / H**0.5
+    b0 = torch.randn(V, device=DEV, generator=gen) * 0.1
+
+    def run(scale, fused_batch_size=None):
+        t = [x.clone().requires_grad_(True) for x in (f0, g0, W0, b0)]
+        costs = joint_rnnt_loss(*t, labels, act_lens, label_lens, cfg.blank, fused_batch_size=fused_batch_size)
+        (costs * scale).sum().backward()
+        return costs.detach(), [x.grad for x in t]
+
+    costs, (df, dg, dW, db) = run(1.0)
+    assert bool(torch.isfinite(costs).all()) and bool((costs > 0).all())
+    for x in (df, dg, dW, db):
+        assert bool(torch.isfinite(x.float()).all())
+    # (2a) a cell's gradient of the logits sums to zero over the vocabulary, so d bias does
+    assert db.abs().max().item() > 1.0 and abs(db.sum().item()) <= 1e-3 * db.abs().sum().item()
+    # (2b) nothing outside the utterances
+    t_idx = torch.arange(T, device=DEV).view(1, T, 1)
+    u_idx = torch.arange(U, device=DEV).view(1, U, 1)
+    assert bool((df[(t_idx >= act_lens.view(B, 1, 1)).expand_as(df)] == 0).all())
+    assert bool((dg[(u_idx > label_lens.view(B, 1, 1)).expand_as(dg)] == 0).all())
+    # (2c) linear in grad_output (a power of two: exact up to the bf16 roundings' own scaling)
+    costs2, (df2, dg2, dW2, db2) = run(2.0)
+    assert torch.equal(costs2, costs)
+    for a, b in ((df, df2), (dg, dg2), (dW, dW2), (db, db2)):
+        assert (2 * a.float() - b.float()).abs().max().item() <= 2.0**-7 * b.float().abs().max().item()
+    # (2d) sub-batches
+    costs4, (df4, dg4, dW4, db4) = run(1.0, fused_batch_size=4)
+    assert torch.equal(costs4, costs) and torch.equal(df4, df) and torch.equal(dg4, dg)
+    for a, b in ((dW, dW4), (db, db4)):
+        assert (a - b).abs().max().item() <= 1e-4 * a.abs().max().item()
+    # (1) the smallest utterance against the oracle
+    b = int((act_lens * (label_lens + 1)).argmin())
+    tb, ub = int(act_lens[b]), int(label_lens[b]) + 1
+    ref = oracle.joint_rnnt_loss(f0[b : b + 1, :tb].float().cpu().numpy(), g0[b : b + 1, :ub].float().cpu().numpy(),
+                                 W0.cpu().numpy(), b0.cpu().numpy(), labels[b : b + 1, : ub - 1].cpu().numpy(), [tb],
+                                 [ub - 1], cfg.blank)  # fmt: skip
+    np.testing.assert_allclose(costs[b].item(), ref[0][0], rtol=COST_RTOL)
+    for got, want in ((df[b, :tb], ref[1][0]), (dg[b, :ub], ref[2][0])):
+        err = np.abs(got.float().cpu().numpy() - want).max()
+        assert err <= 2.0**-6 * np.abs(want).max() + 1e-7, err

@@ -1,10 +1,11 @@
-"""GPU parity of the fused joint + RNNT loss (mi_joint_rnnt_forward / mi_joint_rnnt_backward_logits through
-speech_amd.joint) against oracle.joint_rnnt_loss.
+"""GPU parity of the fused joint + RNNT loss (mi_joint_rnnt_forward / mi_joint_rnnt_backward / mi_joint_reduce_hidden
+through speech_amd.joint) against oracle.joint_rnnt_loss.
 
 Tolerances.  Costs: 1e-5 relative (the bar of the loss itself; float32 accumulation against the oracle's exact
-sums of the same bf16 operands).  Gradients: the kernel stores the gradient of the logits as bf16 and the two GEMMs
-return bf16, as the reference's autocast backward does (two roundings of 2^-9 each on every term of the sums over u
-and t, whose terms may cancel), so each gradient tensor is held to 2^-6 of its own largest entry."""
+sums of the same bf16 operands).  Gradients: the backward forms the probabilities from the fp16 copy of the logits
+the forward kept (2^-11 relative on a logit) and rounds the gradient of the logits and d hidden to bf16, as the
+reference's autocast backward does (roundings of 2^-9 on every term of the sums over u and t, whose terms may cancel),
+so each gradient tensor is held to 2^-6 of its own largest entry."""
 
 import numpy as np
 import pytest
@@ -204,3 +205,97 @@ def test_dropout_seed_follows_torch_manual_seed():
     assert torch.equal(a, c) and not torch.equal(a, b)
     with pytest.raises(ValueError):
         joint_rnnt_forward(*args, dropout=1.0)
+
+
+def test_backward_leaves_what_the_forward_kept_and_serves_any_subset_of_the_inputs():
+    """The backward only reads the saved logits and activations: a second backward through the same graph gives the
+    same gradients bit for bit (the two product kernels and their partial sums have no atomics), and gradients of a
+    subset of the inputs (only f and g: no d weight kernel; only weight and bias: no d hidden kernel, no reductions)
+    equal the ones computed together."""
+    f, g, W, bias, labels, al, ll = make_case(31, 4, 21, 9, 640, 300)
+    lab, ald, lld = dev_ints(labels, al, ll)
+
+    def grads(which):
+        t = [f.to(DEV), g.to(DEV), W.to(DEV), bias.to(DEV)]
+        for i in which:
+            t[i].requires_grad_(True)
+        costs = joint_rnnt_loss(*t, lab, ald, lld, 299, 0.01, 0.0)
+        first = torch.autograd.grad(costs.sum(), [t[i] for i in which], retain_graph=True)
+        second = torch.autograd.grad(costs.sum(), [t[i] for i in which])
+        for a, b in zip(first, second):
+            assert torch.equal(a, b)
+        return dict(zip(which, first))
+
+    every = grads((0, 1, 2, 3))
+    for subset in ((0, 1), (2, 3), (0,), (2,)):
+        for i, x in grads(subset).items():
+            assert torch.equal(x, every[i]), (subset, i)
+
+
+def test_saved_rows_are_sized_by_the_tile_bound_and_checked():
+    """The C entry points: a forward that keeps its logits needs room for every tile lattices without padding would have
+    (both buffers or neither); the backward wants at least one output and its partial-sum buffers together."""
+    import ctypes
+
+    from speech_amd import _native
+    from speech_amd.joint import fused
+
+    lib = _native.lib()
+    B, T, U, H, V = 3, 37, 11, 256, 70
+    assert lib.mi_joint_tile_bound(B, T, U) == B * ((T * U + 127) // 128)
+    assert lib.mi_joint_tile_bound(0, T, U) == 0 and lib.mi_joint_tile_bound(1 << 20, 1 << 15, 1 << 10) == 0
+    f, g, W, bias, labels, al, ll = make_case(32, B, T, U, H, V)
+    fd, gd, Wd, bd = f.to(DEV), g.to(DEV), W.to(DEV), bias.to(DEV)
+    lab, ald, lld = dev_ints(labels, al, ll)
+    ws = fused.joint_workspace(B, T, U, H, V, DEV)
+    tiles = lib.mi_joint_tile_bound(B, T, U)
+    NP = lib.mi_joint_padded_vocabulary(V)
+    costs = torch.empty(B, device=DEV)
+    logits = torch.empty(tiles * 128, NP, dtype=torch.float16, device=DEV)
+    acts = torch.empty(tiles * 128, H + 16, dtype=torch.bfloat16, device=DEV)
+    stream = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+
+    def forward(lg, ac, n):
+        return lib.mi_joint_rnnt_forward(
+            fd.data_ptr(), gd.data_ptr(), Wd.data_ptr(), bd.data_ptr(), _native.DTYPE_F32, lab.data_ptr(), ald.data_ptr(),
+            lld.data_ptr(), costs.data_ptr(), None, 0.0, 0, 0, B, T, U, H, V, V - 1, 0.0, 1, lg, ac, n, ws.data_ptr(),
+            ws.numel(), stream)  # fmt: skip
+
+    assert forward(logits.data_ptr(), acts.data_ptr(), tiles - 1) == _native.INVALID_VALUE
+    assert forward(logits.data_ptr(), None, tiles) == _native.INVALID_VALUE
+    assert forward(None, acts.data_ptr(), tiles) == _native.INVALID_VALUE
+    assert forward(logits.data_ptr(), acts.data_ptr(), tiles) == _native.SUCCESS
+    torch.cuda.synchronize()
+    want = joint_rnnt_forward(fd, gd, Wd, bd, lab, ald, lld, V - 1)
+    assert torch.equal(costs, want)
+    # the saved logits are the logits: row r of tile order is cell (t, u) = divmod(r - first row of b, U_b)
+    hidden = torch.relu(fd.unsqueeze(2) + gd.unsqueeze(1)).float()
+    full = hidden @ Wd.to(torch.bfloat16).float().t() + bd
+    row0 = 0
+    for b in range(B):
+        Tb, Ub = int(al[b]), int(ll[b]) + 1
+        got = logits[row0 : row0 + Tb * Ub, :V].float().view(Tb, Ub, V)
+        assert (got - full[b, :Tb, :Ub]).abs().max().item() <= 2.0**-10 * full[b, :Tb, :Ub].abs().max().item() + 1e-6
+        assert torch.equal(acts[row0 : row0 + Tb * Ub, :H].view(Tb, Ub, H).float(), hidden[b, :Tb, :Ub].to(torch.bfloat16).float())
+        assert torch.all(logits[row0 : row0 + Tb * Ub, V:NP] == float("-inf"))
+        row0 += -(-Tb * Ub // 128) * 128
+    d_hidden = torch.empty(tiles * 128, H, dtype=torch.bfloat16, device=DEV)
+    slices = 4
+    dw = torch.empty(slices, NP, H, device=DEV)
+    db = torch.empty(slices, NP, device=DEV)
+
+    def backward(dh, a, w, bpart, n):
+        return lib.mi_joint_rnnt_backward(
+            lab.data_ptr(), ald.data_ptr(), lld.data_ptr(), logits.data_ptr(), a, dh, w, bpart, n, tiles, None, 0, 1.0, B, T,
+            U, H, V, V - 1, 0.0, 0.0, ws.data_ptr(), ws.numel(), stream)  # fmt: skip
+
+    assert backward(None, None, None, None, slices) == _native.INVALID_VALUE                      # nothing wanted
+    assert backward(None, None, dw.data_ptr(), db.data_ptr(), slices) == _native.INVALID_VALUE    # d weight needs the activations
+    assert backward(None, acts.data_ptr(), dw.data_ptr(), None, slices) == _native.INVALID_VALUE  # and both partial buffers
+    assert backward(None, acts.data_ptr(), dw.data_ptr(), db.data_ptr(), 0) == _native.INVALID_VALUE
+    assert backward(d_hidden.data_ptr(), acts.data_ptr(), dw.data_ptr(), db.data_ptr(), slices) == _native.SUCCESS
+    torch.cuda.synchronize()
+    # the column sums of d weight's operands: d bias = sum over the cells of the gradient of the logits, which sums
+    # to (1 - 1) = 0 over a cell's vocabulary without FastEmit: the whole vector sums to ~0 against entries of order 1
+    bias_grad = db.sum(0)[:V]
+    assert bias_grad.abs().max().item() > 0.1 and abs(bias_grad.sum().item()) < 1e-2 * bias_grad.abs().sum().item()

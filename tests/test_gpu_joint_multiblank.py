@@ -1,4 +1,4 @@
-"""GPU parity of the fused joint + multi-blank loss (mi_joint_multiblank_forward / _backward_logits through
+"""GPU parity of the fused joint + multi-blank loss (mi_joint_multiblank_forward / _backward through
 speech_amd.joint) against oracle.joint_rnnt_loss(..., big_blank_durations=...): the big blanks are ordinary outputs
 of the joint's Linear layer at blank-1-i (rnnt_pytorch.py:442-510).  Tolerances as in tests/test_gpu_joint.py."""
 

@@ -1,9 +1,10 @@
-"""GPU parity of the fused joint + TDT loss (mi_joint_tdt_forward / mi_joint_tdt_backward_logits through
+"""GPU parity of the fused joint + TDT loss (mi_joint_tdt_forward / mi_joint_tdt_backward through
 speech_amd.joint) against oracle.joint_rnnt_loss(..., durations=...): the joint's Linear layer has V + D outputs, the
 token logits followed by the duration logits (rnnt_pytorch.py:563-568).
 
 Tolerances as for the RNNT variant (tests/test_gpu_joint.py): costs 1e-5 relative; every gradient tensor within 2^-6
-of its own largest entry (the gradient of the logits and the two GEMM results are bf16, as in autocast)."""
+of its own largest entry (the gradient of the logits and d hidden are bf16, as in autocast; the probabilities come from an
+fp16 copy of the logits)."""
 
 import random
 
