@@ -72,3 +72,78 @@ def test_tdt_forward_backward_in_a_graph():
 
 def test_multiblank_forward_backward_in_a_graph():
     eager_and_graph("multiblank", 3, 17, 6, 40, {"big": [2, 4]}, 3)
+
+
+def test_fused_joint_forward_and_backward_replay_from_a_graph():
+    """The fused joint's step reads nothing back from the device (its row buffers are sized by a bound the host
+    knows, the tiles in use are counted and consumed on the device), so the C-level forward, backward and reduction
+    can be captured and replayed on new inputs -- with other lengths, i.e. another number of tiles in use."""
+    import ctypes
+
+    from speech_amd import _native
+    from speech_amd.joint import fused
+
+    lib = _native.lib()
+    B, T, U, H, V = 4, 23, 9, 640, 130
+    rng = np.random.RandomState(5)
+    f = torch.zeros(B, T, H, dtype=torch.bfloat16, device=DEV)
+    g = torch.zeros(B, U, H, dtype=torch.bfloat16, device=DEV)
+    W = torch.tensor(rng.randn(V, H) / np.sqrt(H), dtype=torch.float32, device=DEV)
+    bias = torch.tensor(rng.randn(V) * 0.3, dtype=torch.float32, device=DEV)
+    labels = torch.tensor(rng.randint(0, V - 1, size=(B, U - 1)), device=DEV)
+    al = torch.full((B,), T, dtype=torch.int64, device=DEV)
+    ll = torch.full((B,), U - 1, dtype=torch.int64, device=DEV)
+    ws = fused.joint_workspace(B, T, U, H, V, DEV)
+    tiles = lib.mi_joint_tile_bound(B, T, U)
+    NP = lib.mi_joint_padded_vocabulary(V)
+    slices = 8
+    logits = torch.empty(tiles * 128, NP, dtype=torch.float16, device=DEV)
+    acts = torch.empty(tiles * 128, H + 16, dtype=torch.bfloat16, device=DEV)
+    d_hidden = torch.empty(tiles * 128, H, dtype=torch.bfloat16, device=DEV)
+    scale = torch.ones(B, device=DEV)
+
+    def run(out):
+        costs, dw, db, df, dg = out
+        stream = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+        args = (B, T, U, H, V, V - 1)
+        st = lib.mi_joint_rnnt_forward(f.data_ptr(), g.data_ptr(), W.data_ptr(), bias.data_ptr(), _native.DTYPE_F32,
+                                       labels.data_ptr(), al.data_ptr(), ll.data_ptr(), costs.data_ptr(), None, 0.0, 0, 0,
+                                       *args, 0.01, 1, logits.data_ptr(), acts.data_ptr(), tiles, ws.data_ptr(),
+                                       ws.numel(), stream)  # fmt: skip
+        assert st == _native.SUCCESS
+        st = lib.mi_joint_rnnt_backward(labels.data_ptr(), al.data_ptr(), ll.data_ptr(), logits.data_ptr(), acts.data_ptr(),
+                                        d_hidden.data_ptr(), dw.data_ptr(), db.data_ptr(), slices, tiles, scale.data_ptr(),
+                                        1, 1.0, *args, 0.01, 0.0, ws.data_ptr(), ws.numel(), stream)  # fmt: skip
+        assert st == _native.SUCCESS
+        st = lib.mi_joint_reduce_hidden(d_hidden.data_ptr(), f.data_ptr(), g.data_ptr(), al.data_ptr(), ll.data_ptr(),
+                                        df.data_ptr(), dg.data_ptr(), tiles, 0.0, 0, 0, B, T, U, H, V, 0, 0, ws.data_ptr(),
+                                        ws.numel(), stream)  # fmt: skip
+        assert st == _native.SUCCESS
+
+    def outputs():
+        return (torch.empty(B, device=DEV), torch.empty(slices, NP, H, device=DEV), torch.empty(slices, NP, device=DEV),
+                torch.empty(B, T, H, device=DEV), torch.empty(B, U, H, device=DEV))
+
+    eager, captured = outputs(), outputs()
+    f.copy_(torch.tensor(rng.randn(B, T, H), dtype=torch.bfloat16))
+    g.copy_(torch.tensor(rng.randn(B, U, H), dtype=torch.bfloat16))
+    run(eager)  # warm-up outside the capture
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        run(captured)
+    for replay in range(4):
+        f.copy_(torch.tensor(rng.randn(B, T, H) * (1 + 0.5 * replay), dtype=torch.bfloat16))
+        g.copy_(torch.tensor(rng.randn(B, U, H), dtype=torch.bfloat16))
+        a, l = make_lengths(rng, B, T, U, 2, 0)
+        al.copy_(torch.tensor(a))
+        ll.copy_(torch.tensor(l))
+        scale.copy_(torch.tensor(rng.rand(B) + 0.5, dtype=torch.float32))
+        for x in captured:
+            x.fill_(-3.0)
+        graph.replay()
+        torch.cuda.synchronize()
+        run(eager)  # the program's own eager work between replays
+        torch.cuda.synchronize()
+        for name, x, y in zip(("costs", "dw", "db", "df", "dg"), captured, eager):
+            assert torch.equal(x, y), (name, replay)
