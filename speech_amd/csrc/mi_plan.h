@@ -38,11 +38,16 @@ inline int prefill_log_rows(size_t row_bytes) {
 // ----------------------------------------------------------------------------------------
 // Workspace layout
 // ----------------------------------------------------------------------------------------
+// A cell's arc log-probs are one record of consecutive floats -- blank, label, then the `extras` duration (TDT) or
+// big-blank (multi-blank) log-probs -- so that the pass that forms them writes them with one store: 2 floats, or a
+// multiple of 4 (whole 16-byte pieces) when there are extras.
+constexpr int arc_record_floats(int extras) { return extras <= 0 ? 2 : (2 + extras + 3) / 4 * 4; }
+
 struct Layout {
   int K;    // lattice cells per lane (1,2,4,8,16)
   int Us;   // pitch of a skewed lattice row = 64*K >= U
   int ND;   // number of anti-diagonals of the padded lattice = T+U-1
-  int A;    // arc planes per diagonal row: blank, label, D duration log-probs
+  int A;    // floats of a cell's record of arc log-probs (arc_record_floats); a skewed row holds Us records
   int CS;   // floats per cell in the coefficient buffer
   size_t off_denom, off_arcs, off_alphas, off_betas, off_ll, off_coef, off_fill, total;
 };
@@ -56,7 +61,7 @@ inline bool make_layout(int B, int T, int U, int D, Layout* L) {
   L->K = K;
   L->Us = 64 * K;
   L->ND = T + U - 1;
-  L->A = 2 + D;
+  L->A = arc_record_floats(D);
   L->CS = kCoefBase + ((D + 3) & ~3);
   const size_t cells = (size_t)B * T * U;
   const size_t skew = (size_t)B * L->ND * L->Us;

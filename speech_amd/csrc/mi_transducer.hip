@@ -3,8 +3,9 @@
 // Pipeline of a forward + backward call (one stream, no host synchronisation, nothing allocated):
 //   pass 1   denom_rows_kernel | denom_block_kernel | denom_gather_kernel      (mi_streaming.inc)
 //            streams the valid rows of acts once (16-byte aligned loads, log-sum-exp per row) and leaves per
-//            cell the denominator and the blank / label (/ duration / big-blank) log-probabilities in a SKEWED
-//            layout [b][t+u][plane][u], so that an anti-diagonal of the lattice is contiguous.
+//            cell the denominator and, as one record of consecutive floats, the blank / label (/ duration /
+//            big-blank) log-probabilities, the records in a SKEWED layout [b][t+u][u][record], so that an
+//            anti-diagonal of the lattice is contiguous and a cell's record leaves in one store.
 //   lattice  rnnt_lattice_kernel | tdt_lattice_pair_kernel | tdt_lattice_kernel  (mi_lattice.inc)
 //            | multiblank_lattice_kernel | multiblank_lattice_pull_kernel        (mi_multiblank.inc)
 //            alpha and beta over the anti-diagonals, accumulated in fp64 (only the log1p(exp(.)) term in fp32);
