@@ -356,11 +356,15 @@ int mi_joint_multiblank_backward(const int64_t* labels, const int64_t* act_lens,
  * activation's derivative, summed over u into d_f [B,T,H] and over t into d_g [B,U,H] (float32; either may be NULL; frames
  * and label positions outside an utterance get zeros).  The derivative is recomputed from f and g (the forward
  * call's bf16 inputs), `tiles` is the same count as in mi_joint_rnnt_backward, the workspace the forward
- * call's. */
+ * call's.
+ * With dg_part (float32 [chunks][B][U][H], 1 <= chunks <= T; U <= 256; d_g NULL, d_f not) both sums are formed in ONE
+ * pass over d_hidden instead of one pass each: d_f as above, and for each of `chunks` runs of frames the run's share of
+ * d g, which the caller adds up (d g = the sum of dg_part over its first axis; a fixed order of addition keeps the
+ * result the same from call to call). */
 int mi_joint_reduce_hidden(const void* d_hidden, const void* f, const void* g, const int64_t* act_lens,
-                           const int64_t* label_lens, float* d_f, float* d_g, int tiles, float dropout_p,
-                           unsigned long long dropout_seed, int activation, int B, int T, int U, int H, int V, int D,
-                           int num_big_blanks, void* workspace, size_t workspace_bytes, void* stream);
+                           const int64_t* label_lens, float* d_f, float* d_g, float* dg_part, int chunks, int tiles,
+                           float dropout_p, unsigned long long dropout_seed, int activation, int B, int T, int U, int H,
+                           int V, int D, int num_big_blanks, void* workspace, size_t workspace_bytes, void* stream);
 
 /* Where the forward call left the packed weights inside its workspace: *rows x *pitch bf16, row n = weight[n, :]
  * followed by the bias columns (rows beyond V + D are zero in the first H columns), so that the d_hidden product

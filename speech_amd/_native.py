@@ -21,7 +21,7 @@ CPU_SOURCES = [os.path.join(CSRC_DIR, "mi_cpu.cpp")]
 CPU_ABI_VERSION = 1
 CXX_FLAGS = ["-O3", "-std=c++17", "-fPIC", "-shared", "-fopenmp", "-Wall", "-Wextra"]
 
-ABI_VERSION = 19
+ABI_VERSION = 20
 SUCCESS, INVALID_VALUE, LAUNCH_FAILURE, TOO_LARGE = 0, 1, 2, 3
 STATIC_WORKSPACE_BYTES = 64 << 20
 DTYPE_F32, DTYPE_BF16, DTYPE_F16 = 0, 1, 2
@@ -131,8 +131,8 @@ _SIGNATURES = {
     "mi_joint_multiblank_backward": [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _c_int, ctypes.c_longlong, _vp, _c_int,
                                      _c_float, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _vp, _c_int, _c_float,
                                      _c_float, _c_float, _vp, _c_size_t, _vp],
-    "mi_joint_reduce_hidden": [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _c_int, _c_float, ctypes.c_uint64, _c_int, _c_int, _c_int,
-                               _c_int, _c_int, _c_int, _c_int, _c_int, _vp, _c_size_t, _vp],
+    "mi_joint_reduce_hidden": [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _c_int, _c_int, _c_float, ctypes.c_uint64, _c_int,
+                               _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _vp, _c_size_t, _vp],
     "mi_joint_packed_weights": [_vp, _c_size_t, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int,
                                 ctypes.POINTER(_vp),
                                 ctypes.POINTER(_c_int), ctypes.POINTER(_c_int)],

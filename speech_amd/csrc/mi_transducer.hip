@@ -66,7 +66,7 @@ namespace {
 // ----------------------------------------------------------------------------------------
 extern "C" {
 
-int mi_transducer_abi_version(void) { return 19; }
+int mi_transducer_abi_version(void) { return 20; }
 
 int mi_transducer_workspace_bytes(int B, int T, int U, int D, size_t* out_bytes) {
   Layout L;

@@ -116,8 +116,8 @@ def test_fused_joint_forward_and_backward_replay_from_a_graph():
                                         1, 1.0, *args, 0.01, 0.0, ws.data_ptr(), ws.numel(), stream)  # fmt: skip
         assert st == _native.SUCCESS
         st = lib.mi_joint_reduce_hidden(d_hidden.data_ptr(), f.data_ptr(), g.data_ptr(), al.data_ptr(), ll.data_ptr(),
-                                        df.data_ptr(), dg.data_ptr(), tiles, 0.0, 0, 0, B, T, U, H, V, 0, 0, ws.data_ptr(),
-                                        ws.numel(), stream)  # fmt: skip
+                                        df.data_ptr(), dg.data_ptr(), None, 0, tiles, 0.0, 0, 0, B, T, U, H, V, 0, 0,
+                                        ws.data_ptr(), ws.numel(), stream)  # fmt: skip
         assert st == _native.SUCCESS
 
     def outputs():
