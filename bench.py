@@ -48,11 +48,11 @@ HBM_PEAK_GBPS = 8000.0  # MI355X HBM3E, published peak
 MEASURED_TRAFFIC_KIB = {
     # workload: (FETCH_SIZE, WRITE_SIZE) of the gradient-pass kernel in KiB per dispatch; the factors below are what the
     # same counters need to read a 1 GiB copy right (profiles/transducer_kernels_<cfg>_hbm_traffic.md)
-    "cfg2_rnnt_B16_T375_U121_V1025_f32": (807556, 2584313),
-    "cfg3_rnnt_B32_T750_U201_V1025_bf16": (2938561, 8579888),
-    "cfg4_tdt_B16_T375_U121_V1025_D5_f32": (760703, 1780017),
-    "cfg5_rnnt_B8_T250_U101_V16385_f32": (3669515, 12792561),
-    "cfg6_multiblank_B16_T375_U121_V1028_f32": (684910, 1975139),
+    "cfg2_rnnt_B16_T375_U121_V1025_f32": (807541, 2598715),
+    "cfg3_rnnt_B32_T750_U201_V1025_bf16": (2938583, 8566134),
+    "cfg4_tdt_B16_T375_U121_V1025_D5_f32": (760714, 1786097),
+    "cfg5_rnnt_B8_T250_U101_V16385_f32": (3669187, 12770381),
+    "cfg6_multiblank_B16_T375_U121_V1028_f32": (684890, 1978605),
 }
 TRAFFIC_SCALE = (2.0, 1.0)
 

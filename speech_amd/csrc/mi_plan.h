@@ -39,9 +39,10 @@ inline int prefill_log_rows(size_t row_bytes) {
 // Workspace layout
 // ----------------------------------------------------------------------------------------
 // A cell's arc log-probs are one record of consecutive floats -- blank, label, then the `extras` duration (TDT) or
-// big-blank (multi-blank) log-probs -- so that the pass that forms them writes them with one store: 2 floats, or a
-// multiple of 4 (whole 16-byte pieces) when there are extras.
-constexpr int arc_record_floats(int extras) { return extras <= 0 ? 2 : (2 + extras + 3) / 4 * 4; }
+// big-blank (multi-blank) log-probs -- so that the pass that forms them writes them with one store: 2 floats, or,
+// when there are extras, a multiple of 4 (whole 16-byte pieces) whose LAST float is the cell's log-softmax
+// denominator (the cell kernels of those losses read it there, and the pass saves the store into `denom`).
+constexpr int arc_record_floats(int extras) { return extras <= 0 ? 2 : (3 + extras + 3) / 4 * 4; }
 
 struct Layout {
   int K;    // lattice cells per lane (1,2,4,8,16)

@@ -393,8 +393,8 @@ int mi_transducer_export_lattice(const void* workspace, size_t workspace_bytes, 
   hipLaunchKernelGGL(export_lattice_kernel, dim3(grid), dim3(256), 0, (hipStream_t)stream,
                      (const float*)(ws + L.off_denom), (const double*)(ws + L.off_alphas),
                      (const double*)(ws + L.off_betas), (const double*)(ws + L.off_ll),
-                     act_lens, label_lens, denom, alphas, betas,
-                     ll_forward, ll_backward, B, T, U, L.ND, L.Us, cells);
+                     (const float*)(ws + L.off_arcs), act_lens, label_lens, denom, alphas, betas,
+                     ll_forward, ll_backward, B, T, U, L.ND, L.Us, L.A, cells);
   return launch_status();
 }
 

@@ -55,7 +55,7 @@ static void fuzz_plan(std::mt19937& rng, int iterations) {
       const size_t offs[] = {L.off_denom, L.off_arcs, L.off_alphas, L.off_betas, L.off_ll,
                              L.off_coef,  L.off_fill, L.total};
       for (int i = 0; i + 1 < 8; ++i) EXPECT(offs[i] < offs[i + 1] && (offs[i] & 255) == 0, "segment %d", i);
-      EXPECT(L.Us >= U && L.Us == 64 * L.K && L.ND == T + U - 1 && L.A >= 2 + D && L.A == arc_record_floats(D) && (D == 0 ? L.A == 2 : L.A % 4 == 0 && L.A < 2 + D + 4) && L.CS >= kCoefBase + D, "layout");
+      EXPECT(L.Us >= U && L.Us == 64 * L.K && L.ND == T + U - 1 && L.A >= 2 + D && L.A == arc_record_floats(D) && (D == 0 ? L.A == 2 : L.A % 4 == 0 && L.A >= 3 + D && L.A < 3 + D + 4) && L.CS >= kCoefBase + D, "layout");
       const size_t cells = (size_t)B * T * U, skew = (size_t)B * L.ND * L.Us;
       EXPECT(L.off_arcs - L.off_denom >= cells * 4 && L.off_alphas - L.off_arcs >= skew * L.A * 4 &&
                  L.off_betas - L.off_alphas >= skew * 8 && L.off_ll - L.off_betas >= skew * 8 &&
